@@ -1,0 +1,225 @@
+"""Benchmark of the fused camera->BEV pooling on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--table]
+
+One step = one forward plus one backward pass of the operator over one batch of seeded
+synthetic input that is already resident in HBM: forward kernel, zero-fill of the two
+gradient buffers, backward kernel, all queued on PyTorch's current stream through the
+extension module.  The default workload is the 6-camera 128x128x8 fp32 configuration
+(``cfg2_surround``) with the reference benchmark's depth model (per-pixel Laplace
+parameters, tools/config/config.yaml:29).  The single JSON line printed on stdout carries
+  value / ms_per_step   forward+backward latency per step (ms)
+  roofline              dominant kernel: compulsory bytes of that kernel / its mean duration
+                        (HIP events recorded around every launch in the timed region),
+                        against the 8 TB/s HBM3E peak
+  cpu_baseline          the dense PyTorch restatement of the reference's pooling path
+                        (oracle/dense_torch.py), forward+backward via autograd on the host
+                        cores, same workload -- a reported baseline, not a target.
+``--table`` additionally measures every configuration and depth model, forward and
+forward+backward, and writes the table to gpurun_out/bench_table.{json,md}.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from flashbev_amd._native import load_ext  # noqa: E402
+from flashbev_amd.flash_bevpool import voxel_geometry  # noqa: E402
+from flashbev_amd.workloads import WORKLOADS, algorithmic_bytes, make_inputs  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+DIST_OF = {"gaussian": (0, "parametric"), "laplace": (1, "parametric"), "categorical": (2, "categorical")}
+
+
+class Runner:
+    """Pre-allocated buffers and the four queued operations of one step."""
+
+    def __init__(self, w, depth_name: str, device: str = "cuda:0"):
+        self.w = w
+        self.dist, self.model = DIST_OF[depth_name]
+        self.ext = load_ext()
+        x = make_inputs(w, self.model, device=device, with_grad_out=True)
+        self.x = x
+        B, N, H, W, C = x["image_feats"].shape
+        gx, gy, gz = w.grid_size
+        self.out = torch.empty((B, gy, gx, C), dtype=torch.float32, device=device)
+        self.d_depth = torch.zeros(x["depth_params"].shape, dtype=torch.float32, device=device)
+        self.d_feats = torch.zeros(x["image_feats"].shape, dtype=torch.float32, device=device)
+        self.vmin, self.vsize = voxel_geometry(w.roi_range, w.grid_size)
+        self.eps, self.thr = 1e-6, 1e-6
+
+    def forward(self):
+        x, w = self.x, self.w
+        self.ext.flash_bevpool_forward(
+            x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"], x["image_size"],
+            x["grid_size"], self.vsize[0], self.vsize[1], self.vsize[2], self.vmin[0], self.vmin[1],
+            self.vmin[2], self.out, self.out.numel(), self.dist, True, True, False, False, self.eps, self.thr,
+            w.depth_range[0], w.depth_range[1], 0)
+
+    def zero_grads(self):
+        self.d_depth.zero_()
+        self.d_feats.zero_()
+
+    def backward(self):
+        x, w = self.x, self.w
+        self.ext.flash_bevpool_backward(
+            x["grad_out"], x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
+            x["image_size"], x["roi_range"], x["grid_size"], self.d_depth, self.d_feats, self.out.numel(),
+            self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0)
+
+
+def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
+    """Wall-clock over exactly `steps` steps plus per-kernel HIP-event durations."""
+    for _ in range(warmup):
+        r.forward()
+        if with_backward:
+            r.zero_grads()
+            r.backward()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev[i][0].record()
+        r.forward()
+        ev[i][1].record()
+        if with_backward:
+            r.zero_grads()
+            ev[i][2].record()
+            r.backward()
+            ev[i][3].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    fwd = [ev[i][0].elapsed_time(ev[i][1]) for i in range(steps)]
+    bwd = [ev[i][2].elapsed_time(ev[i][3]) for i in range(steps)] if with_backward else []
+    return (t1 - t0) * 1e3 / steps, fwd, bwd
+
+
+def cpu_baseline(w, depth_name: str, budget_s: float = 20.0, max_runs: int = 5):
+    """Dense PyTorch path on the host cores, forward+backward, bounded to ~budget_s."""
+    from oracle import dense_torch
+
+    dist, model = DIST_OF[depth_name]
+    x = make_inputs(w, model, device="cpu", with_grad_out=True)
+    kw = dict(image_size=w.image_hw, roi_range=w.roi_range, grid_size=w.grid_size, depth_distribution=dist,
+              epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=w.depth_range)
+    f, d = x["image_feats"].float(), x["depth_params"].float()
+    cores = torch.get_num_threads()
+    times = []
+    t_start = time.perf_counter()
+    for i in range(max_runs + 1):
+        t0 = time.perf_counter()
+        dense_torch.dense_pool_grads(f, d, x["projection_matrices"], x["grad_out"], **kw)
+        dt = time.perf_counter() - t0
+        if i > 0:
+            times.append(dt)
+        if time.perf_counter() - t_start > budget_s and times:
+            break
+    return {"value": statistics.mean(times) * 1e3, "unit": "ms", "cores": cores, "kind": "port",
+            "sample": f"{w.name} full workload, dense PyTorch path fwd+bwd, 1 warm-up + {len(times)} timed runs"}
+
+
+def stats(v):
+    v = sorted(v)
+    q = lambda p: v[min(len(v) - 1, int(p * len(v)))]
+    return {"mean": statistics.mean(v), "std": statistics.pstdev(v), "min": v[0], "p50": q(0.5), "p95": q(0.95),
+            "p99": q(0.99)}
+
+
+def run_table(steps: int, warmup: int):
+    rows = []
+    jobs = [("cfg1_tiny", None), ("cfg2_surround", None)]
+    jobs += [("cfg3_zsweep", z) for z in (4, 8, 12, 16)]
+    jobs += [("cfg4_hires", None), ("cfg5_train", None)]
+    for name, z in jobs:
+        w = WORKLOADS[name] if z is None else WORKLOADS[name].with_z(z)
+        for depth_name in ("laplace", "gaussian", "categorical"):
+            r = Runner(w, depth_name)
+            bwd_on = True
+            ms, fwd, bwd = time_steps(r, steps, warmup, bwd_on)
+            fb, bb = algorithmic_bytes(w, r.model, False), algorithmic_bytes(w, r.model, True)
+            f_ms, b_ms = statistics.mean(fwd), statistics.mean(bwd)
+            rows.append({
+                "workload": w.name, "depth": depth_name, "dtype": str(w.dtype).replace("torch.", ""),
+                "fwd_ms": f_ms, "bwd_ms": b_ms, "fwd_bwd_ms_wall": ms,
+                "fwd_bytes": fb, "bwd_bytes": bb,
+                "fwd_GBps": fb / f_ms / 1e6, "bwd_GBps": bb / b_ms / 1e6,
+                "fwd_frac_hbm": fb / f_ms / 1e6 / HBM_PEAK_GBS, "bwd_frac_hbm": bb / b_ms / 1e6 / HBM_PEAK_GBS,
+                "fwd_p50_ms": stats(fwd)["p50"], "bwd_p50_ms": stats(bwd)["p50"],
+            })
+            print(f"[table] {w.name:16s} {depth_name:11s} fwd {f_ms*1e3:9.1f} us ({rows[-1]['fwd_frac_hbm']*100:5.1f}% HBM) "
+                  f"bwd {b_ms*1e3:9.1f} us ({rows[-1]['bwd_frac_hbm']*100:5.1f}% HBM)", file=sys.stderr, flush=True)
+            del r
+            torch.cuda.empty_cache()
+    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+    with open(os.path.join(ROOT, "gpurun_out", "bench_table.json"), "w") as fh:
+        json.dump(rows, fh, indent=1)
+    with open(os.path.join(ROOT, "gpurun_out", "bench_table.md"), "w") as fh:
+        fh.write("| workload | depth model | dtype | fwd us | fwd GB/s | fwd % of 8 TB/s | bwd us | bwd GB/s | bwd % of 8 TB/s |\n")
+        fh.write("|---|---|---|---|---|---|---|---|---|\n")
+        for r_ in rows:
+            fh.write(f"| {r_['workload']} | {r_['depth']} | {r_['dtype']} | {r_['fwd_ms']*1e3:.1f} | {r_['fwd_GBps']:.0f} | "
+                     f"{r_['fwd_frac_hbm']*100:.1f} | {r_['bwd_ms']*1e3:.1f} | {r_['bwd_GBps']:.0f} | {r_['bwd_frac_hbm']*100:.1f} |\n")
+    return rows
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2_surround", choices=sorted(WORKLOADS))
+    ap.add_argument("--depth", default="laplace", choices=sorted(DIST_OF))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--table", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU; batch elements are independent, so more GPUs "
+              "would each take a slice of the batch with no exchange. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    w = WORKLOADS[args.workload]
+    r = Runner(w, args.depth)
+    ms, fwd, bwd = time_steps(r, args.steps, args.warmup, True)
+    fwd_ms, bwd_ms = statistics.mean(fwd), statistics.mean(bwd)
+    fb, bb = algorithmic_bytes(w, r.model, False), algorithmic_bytes(w, r.model, True)
+    dominant = "backward" if bwd_ms >= fwd_ms else "forward"
+    k_ms, k_bytes = (bwd_ms, bb) if dominant == "backward" else (fwd_ms, fb)
+    achieved = k_bytes / k_ms / 1e6  # GB/s
+    line = {
+        "metric": "BEV-pool fwd+bwd latency (ms) & effective HBM GB/s, 6 cams 128x128xZ=8, 1 GPU",
+        "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if w.dtype == torch.float32 else str(w.dtype).replace("torch.", ""),
+        "data": "synthetic",
+        "config": {"workload": w.name, "depth_model": args.depth, "batch": w.batch, "cams": w.num_cams,
+                   "channels": w.channels, "feat_hw": list(w.feat_hw), "grid": list(w.grid_size),
+                   "step": "forward kernel + zero-fill of both gradient buffers + backward kernel"},
+        "fwd_kernel_ms": stats(fwd), "bwd_kernel_ms": stats(bwd),
+        "effective_GBps_fwd_bwd": (fb + bb) / ms / 1e6,
+        "frac_hbm_fwd_bwd": (fb + bb) / ms / 1e6 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": f"fbev_{dominant}_kernel", "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": k_bytes, "kernel_ms": k_ms},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(w, args.depth)
+    if args.table:
+        run_table(max(20, args.steps // 4), args.warmup)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

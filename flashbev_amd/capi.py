@@ -1,0 +1,118 @@
+"""ctypes view of the C ABI in ``include/flashbev_hip.h`` (libflashbev_hip.so).
+
+This is the binding a non-torch host would write; the parity tests call the kernels
+through it with raw device pointers.  Loading the library needs the ROCm runtime but no
+GPU; calling a compute entry point needs a GPU.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+from . import _build
+
+FBEV_F32, FBEV_F16, FBEV_BF16 = 0, 1, 2
+FBEV_GAUSSIAN, FBEV_LAPLACE, FBEV_CATEGORICAL = 0, 1, 2
+FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
+
+EXPORTS = ("fbev_forward", "fbev_backward", "fbev_sample_geometry", "fbev_algorithmic_bytes",
+           "fbev_status_string", "fbev_abi_version", "fbev_problem_size")
+
+
+class FbevProblem(ctypes.Structure):
+    _fields_ = [
+        ("batch", ctypes.c_int32), ("num_cams", ctypes.c_int32),
+        ("feat_h", ctypes.c_int32), ("feat_w", ctypes.c_int32), ("channels", ctypes.c_int32),
+        ("image_h", ctypes.c_int32), ("image_w", ctypes.c_int32),
+        ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32), ("grid_z", ctypes.c_int32),
+        ("voxel_min", ctypes.c_float * 3), ("voxel_size", ctypes.c_float * 3),
+        ("epsilon", ctypes.c_float), ("depth_weight_threshold", ctypes.c_float),
+        ("depth_distribution", ctypes.c_int32), ("depth_bins", ctypes.c_int32),
+        ("depth_min", ctypes.c_float), ("depth_step", ctypes.c_float),
+        ("in_dtype", ctypes.c_int32), ("reduction", ctypes.c_int32), ("proj_stride", ctypes.c_int32),
+    ]
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        lib = ctypes.CDLL(_build.HIP_LIB)
+        vp, pp = ctypes.c_void_p, ctypes.POINTER(FbevProblem)
+        lib.fbev_forward.argtypes = [pp, vp, vp, vp, vp, vp]
+        lib.fbev_forward.restype = ctypes.c_int
+        lib.fbev_backward.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp]
+        lib.fbev_backward.restype = ctypes.c_int
+        lib.fbev_sample_geometry.argtypes = [pp, vp, vp, vp, vp, vp]
+        lib.fbev_sample_geometry.restype = ctypes.c_int
+        lib.fbev_algorithmic_bytes.argtypes = [pp, ctypes.c_int]
+        lib.fbev_algorithmic_bytes.restype = ctypes.c_uint64
+        lib.fbev_status_string.argtypes = [ctypes.c_int]
+        lib.fbev_status_string.restype = ctypes.c_char_p
+        lib.fbev_abi_version.restype = ctypes.c_int
+        lib.fbev_problem_size.restype = ctypes.c_size_t
+        if lib.fbev_problem_size() != ctypes.sizeof(FbevProblem):
+            raise ImportError("flashbev_amd.capi: fbev_problem layout mismatch between header and binding")
+        _lib = lib
+    return _lib
+
+
+def make_problem(batch, num_cams, feat_hw, channels, image_hw, grid_size, voxel_min, voxel_size,
+                 depth_distribution=0, depth_bins=2, epsilon=1e-6, depth_weight_threshold=1e-6,
+                 depth_range=(1.0, 1.0), in_dtype=FBEV_F32, reduction=FBEV_REDUCE_MEAN,
+                 proj_stride=12) -> FbevProblem:
+    p = FbevProblem()
+    p.batch, p.num_cams = int(batch), int(num_cams)
+    p.feat_h, p.feat_w = int(feat_hw[0]), int(feat_hw[1])
+    p.channels = int(channels)
+    p.image_h, p.image_w = int(image_hw[0]), int(image_hw[1])
+    p.grid_x, p.grid_y, p.grid_z = (int(v) for v in grid_size)
+    for i in range(3):
+        p.voxel_min[i] = float(voxel_min[i])
+        p.voxel_size[i] = float(voxel_size[i])
+    p.epsilon = float(epsilon)
+    p.depth_weight_threshold = float(depth_weight_threshold)
+    p.depth_distribution = int(depth_distribution)
+    p.depth_bins = int(depth_bins)
+    p.depth_min, p.depth_step = float(depth_range[0]), float(depth_range[1])
+    p.in_dtype = int(in_dtype)
+    p.reduction = int(reduction)
+    p.proj_stride = int(proj_stride)
+    return p
+
+
+def status_string(rc: int) -> str:
+    return load().fbev_status_string(int(rc)).decode()
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what} failed: {status_string(rc)} ({rc})")
+
+
+def _p(ptr: Optional[int]):
+    return ctypes.c_void_p(ptr) if ptr else None
+
+
+def forward(p: FbevProblem, depth_ptr: int, feats_ptr: int, proj_ptr: int, out_ptr: int,
+            stream: int = 0) -> int:
+    return load().fbev_forward(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(proj_ptr), _p(out_ptr),
+                               _p(stream))
+
+
+def backward(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
+             d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], stream: int = 0) -> int:
+    return load().fbev_backward(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
+                                _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), _p(stream))
+
+
+def sample_geometry(p: FbevProblem, proj_ptr: int, mask_ptr: Optional[int], idx_ptr: Optional[int],
+                    frac_ptr: Optional[int], stream: int = 0) -> int:
+    return load().fbev_sample_geometry(ctypes.byref(p), _p(proj_ptr), _p(mask_ptr), _p(idx_ptr),
+                                       _p(frac_ptr), _p(stream))
+
+
+def algorithmic_bytes(p: FbevProblem, backward_pass: bool) -> int:
+    return int(load().fbev_algorithmic_bytes(ctypes.byref(p), int(bool(backward_pass))))

@@ -1,0 +1,269 @@
+// flashbevpool_ext: the torch-facing native module of the fused camera->BEV pooling
+// operator.  It exports the two entry points of the reference's extension with the same
+// names and positional order (flashbev/flashbevpool/src/flash_bevpool.cpp:79-101,168-183,
+// 243-246) and does nothing but validate tensors, select the device and PyTorch's current
+// HIP stream, and call the C ABI of libflashbev_hip.so.  Unlike the reference it checks
+// every argument and raises (c10::Error -> RuntimeError) instead of launching on bad input.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <string>
+#include <vector>
+
+#include "flashbev_hip.h"
+
+namespace {
+
+struct DeviceScope {
+    int prev = -1;
+    explicit DeviceScope(int dev) {
+        TORCH_CHECK(hipGetDevice(&prev) == hipSuccess, "flashbevpool_ext: hipGetDevice failed");
+        if (prev != dev) {
+            TORCH_CHECK(hipSetDevice(dev) == hipSuccess, "flashbevpool_ext: hipSetDevice failed");
+        } else {
+            prev = -1;
+        }
+    }
+    ~DeviceScope() { if (prev >= 0) (void)hipSetDevice(prev); }
+};
+
+int dtype_code(const at::Tensor &t, const char *name) {
+    switch (t.scalar_type()) {
+        case at::kFloat: return FBEV_F32;
+        case at::kHalf: return FBEV_F16;
+        case at::kBFloat16: return FBEV_BF16;
+        default: TORCH_CHECK(false, "flashbevpool_ext: ", name, " must be float32, float16 or bfloat16, got ",
+                             t.scalar_type());
+    }
+    return -1;
+}
+
+// Small integer / float tensors (sizes, ranges) may live on either side; a device tensor
+// costs one synchronous copy, as in the reference (flash_bevpool.cpp:118-124).
+std::vector<int64_t> host_ints(const at::Tensor &t, int64_t n, const char *name) {
+    TORCH_CHECK(t.numel() == n, "flashbevpool_ext: ", name, " must have ", n, " elements, got ", t.numel());
+    at::Tensor h = t.to(at::kCPU, at::kLong).contiguous();
+    return std::vector<int64_t>(h.data_ptr<int64_t>(), h.data_ptr<int64_t>() + n);
+}
+
+std::vector<float> host_floats(const at::Tensor &t, int64_t n, const char *name) {
+    TORCH_CHECK(t.numel() == n, "flashbevpool_ext: ", name, " must have ", n, " elements, got ", t.numel());
+    at::Tensor h = t.to(at::kCPU, at::kFloat).contiguous();
+    return std::vector<float>(h.data_ptr<float>(), h.data_ptr<float>() + n);
+}
+
+void check_dev(const at::Tensor &t, const at::Tensor &ref, const char *name) {
+    TORCH_CHECK(t.is_cuda(), "flashbevpool_ext: ", name, " must be a GPU tensor");
+    TORCH_CHECK(t.device() == ref.device(), "flashbevpool_ext: ", name, " is on ", t.device(), " but depth_params is on ",
+                ref.device());
+    TORCH_CHECK(t.is_contiguous(), "flashbevpool_ext: ", name, " must be contiguous");
+}
+
+// Shapes and dtypes shared by forward and backward.
+fbev_problem describe(const at::Tensor &depth, const at::Tensor &feats, const at::Tensor &proj,
+                      const at::Tensor &feature_size, const at::Tensor &image_size, const at::Tensor &grid_size,
+                      int depth_distribution, float epsilon, float threshold, float depth_min, float depth_step,
+                      int reduction) {
+    TORCH_CHECK(depth.is_cuda(), "flashbevpool_ext: depth_params must be a GPU tensor");
+    TORCH_CHECK(depth.is_contiguous(), "flashbevpool_ext: depth_params must be contiguous");
+    check_dev(feats, depth, "image_feats");
+    check_dev(proj, depth, "projection_matrices");
+    TORCH_CHECK(depth.dim() == 5 && feats.dim() == 5,
+                "flashbevpool_ext: depth_params and image_feats must be [B,N,H,W,*], got ", depth.sizes(), " and ",
+                feats.sizes());
+    for (int d = 0; d < 4; ++d)
+        TORCH_CHECK(depth.size(d) == feats.size(d), "flashbevpool_ext: depth_params ", depth.sizes(),
+                    " and image_feats ", feats.sizes(), " disagree in dimension ", d);
+    TORCH_CHECK(depth.scalar_type() == feats.scalar_type(),
+                "flashbevpool_ext: depth_params and image_feats must share a dtype");
+    TORCH_CHECK(proj.scalar_type() == at::kFloat, "flashbevpool_ext: projection_matrices must be float32");
+    TORCH_CHECK(proj.dim() == 4 && proj.size(0) == depth.size(0) && proj.size(1) == depth.size(1) &&
+                    (proj.size(2) == 3 || proj.size(2) == 4) && proj.size(3) == 4,
+                "flashbevpool_ext: projection_matrices must be [B,N,3,4] or [B,N,4,4], got ", proj.sizes());
+    TORCH_CHECK(depth_distribution >= 0 && depth_distribution <= 2,
+                "flashbevpool_ext: depth_distribution must be 0 (gaussian), 1 (laplace) or 2 (categorical), got ",
+                depth_distribution);
+    if (depth_distribution != FBEV_CATEGORICAL)
+        TORCH_CHECK(depth.size(4) == 2, "flashbevpool_ext: depth_params must be [B,N,H,W,2] (mean, sigma), got ",
+                    depth.sizes());
+
+    fbev_problem p{};
+    p.batch = (int32_t)depth.size(0);
+    p.num_cams = (int32_t)depth.size(1);
+    p.feat_h = (int32_t)depth.size(2);
+    p.feat_w = (int32_t)depth.size(3);
+    p.channels = (int32_t)feats.size(4);
+    p.depth_bins = (int32_t)depth.size(4);
+    p.in_dtype = dtype_code(feats, "image_feats");
+
+    // feature_size [B,N,2] repeats (H, W) of the feature tensor for every camera; it can be
+    // checked for free only when it already lives on the host.
+    TORCH_CHECK(feature_size.numel() == (int64_t)p.batch * p.num_cams * 2,
+                "flashbevpool_ext: feature_size must be [B,N,2], got ", feature_size.sizes());
+    if (!feature_size.is_cuda()) {
+        auto fs = host_ints(feature_size, feature_size.numel(), "feature_size");
+        for (size_t i = 0; i < fs.size(); i += 2)
+            TORCH_CHECK(fs[i] == p.feat_h && fs[i + 1] == p.feat_w, "flashbevpool_ext: feature_size entry (",
+                        fs[i], ",", fs[i + 1], ") differs from the feature tensor's (", p.feat_h, ",", p.feat_w, ")");
+    }
+    auto im = host_ints(image_size, 2, "image_size");
+    auto gs = host_ints(grid_size, 3, "grid_size");
+    TORCH_CHECK(im[0] > 0 && im[1] > 0, "flashbevpool_ext: image_size must be positive");
+    TORCH_CHECK(gs[0] > 0 && gs[1] > 0 && gs[2] > 0, "flashbevpool_ext: grid_size must be positive");
+    p.image_h = (int32_t)im[0];
+    p.image_w = (int32_t)im[1];
+    p.grid_x = (int32_t)gs[0];
+    p.grid_y = (int32_t)gs[1];
+    p.grid_z = (int32_t)gs[2];
+    p.epsilon = epsilon;
+    p.depth_weight_threshold = threshold;
+    p.depth_distribution = depth_distribution;
+    p.depth_min = depth_min;
+    p.depth_step = depth_step;
+    p.reduction = reduction;
+    p.proj_stride = (int32_t)(proj.size(2) * 4);
+    return p;
+}
+
+void raise_on(int rc, const char *what) {
+    TORCH_CHECK(rc == FBEV_OK, "flashbevpool_ext: ", what, " failed: ", fbev_status_string(rc), " (", rc, ")");
+}
+
+}  // namespace
+
+// Same positional order as the reference's flash_bevpool_forward
+// (flashbev/flashbevpool/src/flash_bevpool.cpp:79-101).  The four kernel-variant booleans
+// select nothing here (one kernel serves all); the trailing arguments are extensions.
+void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &image_feats,
+                           const at::Tensor &projection_matrices, const at::Tensor &feature_size,
+                           const at::Tensor &image_size, const at::Tensor &grid_size, float voxel_size_x,
+                           float voxel_size_y, float voxel_size_z, float voxel_x_min, float voxel_y_min,
+                           float voxel_z_min, at::Tensor out, int64_t total_threads, int depth_distribution,
+                           bool use_shared_memory, bool optimize_z_precompute, bool use_warp_kernel,
+                           bool use_vectorized_load, float epsilon, float depth_weight_threshold,
+                           float depth_min, float depth_step, int reduction) {
+    (void)use_shared_memory; (void)optimize_z_precompute; (void)use_warp_kernel; (void)use_vectorized_load;
+    fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
+    p.voxel_min[0] = voxel_x_min; p.voxel_min[1] = voxel_y_min; p.voxel_min[2] = voxel_z_min;
+    p.voxel_size[0] = voxel_size_x; p.voxel_size[1] = voxel_size_y; p.voxel_size[2] = voxel_size_z;
+    check_dev(out, depth_params, "out");
+    TORCH_CHECK(out.scalar_type() == at::kFloat, "flashbevpool_ext: out must be float32");
+    TORCH_CHECK(out.dim() == 4 && out.size(0) == p.batch && out.size(1) == p.grid_y && out.size(2) == p.grid_x &&
+                    out.size(3) == p.channels,
+                "flashbevpool_ext: out must be [B,grid_y,grid_x,C] = [", p.batch, ",", p.grid_y, ",", p.grid_x, ",",
+                p.channels, "], got ", out.sizes());
+    TORCH_CHECK(total_threads == out.numel(), "flashbevpool_ext: total_threads (", total_threads,
+                ") must equal out.numel() (", out.numel(), ")");
+    DeviceScope scope(depth_params.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
+    raise_on(fbev_forward(&p, depth_params.data_ptr(), image_feats.data_ptr(), projection_matrices.data_ptr<float>(),
+                          out.data_ptr<float>(), st),
+             "fbev_forward");
+}
+
+// Same positional order as the reference's flash_bevpool_backward
+// (flashbev/flashbevpool/src/flash_bevpool.cpp:168-183).  Gradient buffers are float32 and
+// zero-filled by the caller; an undefined (None) gradient tensor skips that gradient.
+void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_params, const at::Tensor &image_feats,
+                            const at::Tensor &projection_matrices, const at::Tensor &feature_size,
+                            const at::Tensor &image_size, const at::Tensor &roi_range, const at::Tensor &grid_size,
+                            std::optional<at::Tensor> depth_params_grad, std::optional<at::Tensor> image_feats_grad,
+                            int64_t total_threads, int depth_distribution, float epsilon, float depth_weight_threshold,
+                            float depth_min, float depth_step, int reduction) {
+    fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
+    auto roi = host_floats(roi_range, 6, "roi_range");
+    const int32_t g[3] = {p.grid_x, p.grid_y, p.grid_z};
+    for (int a = 0; a < 3; ++a) {
+        p.voxel_min[a] = roi[2 * a];
+        volatile float extent = roi[2 * a + 1] - roi[2 * a];   // one rounded fp32 subtraction
+        p.voxel_size[a] = extent / (float)g[a];                // one rounded fp32 division
+    }
+    check_dev(out_grad, depth_params, "out_grad");
+    TORCH_CHECK(out_grad.scalar_type() == at::kFloat, "flashbevpool_ext: out_grad must be float32");
+    TORCH_CHECK(out_grad.dim() == 4 && out_grad.size(0) == p.batch && out_grad.size(1) == p.grid_y &&
+                    out_grad.size(2) == p.grid_x && out_grad.size(3) == p.channels,
+                "flashbevpool_ext: out_grad must be [B,grid_y,grid_x,C], got ", out_grad.sizes());
+    TORCH_CHECK(total_threads == out_grad.numel(), "flashbevpool_ext: total_threads (", total_threads,
+                ") must equal out_grad.numel() (", out_grad.numel(), ")");
+    float *dd = nullptr, *df = nullptr;
+    if (depth_params_grad.has_value() && depth_params_grad->defined()) {
+        check_dev(*depth_params_grad, depth_params, "depth_params_grad");
+        TORCH_CHECK(depth_params_grad->scalar_type() == at::kFloat && depth_params_grad->sizes() == depth_params.sizes(),
+                    "flashbevpool_ext: depth_params_grad must be float32 with the shape of depth_params");
+        dd = depth_params_grad->data_ptr<float>();
+    }
+    if (image_feats_grad.has_value() && image_feats_grad->defined()) {
+        check_dev(*image_feats_grad, depth_params, "image_feats_grad");
+        TORCH_CHECK(image_feats_grad->scalar_type() == at::kFloat && image_feats_grad->sizes() == image_feats.sizes(),
+                    "flashbevpool_ext: image_feats_grad must be float32 with the shape of image_feats");
+        df = image_feats_grad->data_ptr<float>();
+    }
+    DeviceScope scope(depth_params.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
+    raise_on(fbev_backward(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                           projection_matrices.data_ptr<float>(), dd, df, st),
+             "fbev_backward");
+}
+
+// Parity hook: per-sample validity mask and bilinear corner indices, [B,gy,gx,N,gz(,4|2)].
+std::vector<at::Tensor> sample_geometry(const at::Tensor &projection_matrices, int64_t feat_h, int64_t feat_w,
+                                        int64_t image_h, int64_t image_w, std::vector<int64_t> grid_size,
+                                        std::vector<double> voxel_min, std::vector<double> voxel_size, float epsilon) {
+    TORCH_CHECK(projection_matrices.is_cuda() && projection_matrices.is_contiguous() &&
+                    projection_matrices.scalar_type() == at::kFloat && projection_matrices.dim() == 4 &&
+                    (projection_matrices.size(2) == 3 || projection_matrices.size(2) == 4) &&
+                    projection_matrices.size(3) == 4,
+                "flashbevpool_ext: projection_matrices must be a contiguous float32 GPU tensor [B,N,3|4,4]");
+    TORCH_CHECK(grid_size.size() == 3 && voxel_min.size() == 3 && voxel_size.size() == 3,
+                "flashbevpool_ext: grid_size, voxel_min and voxel_size need 3 entries each");
+    fbev_problem p{};
+    p.batch = (int32_t)projection_matrices.size(0);
+    p.num_cams = (int32_t)projection_matrices.size(1);
+    p.feat_h = (int32_t)feat_h; p.feat_w = (int32_t)feat_w;
+    p.image_h = (int32_t)image_h; p.image_w = (int32_t)image_w;
+    p.grid_x = (int32_t)grid_size[0]; p.grid_y = (int32_t)grid_size[1]; p.grid_z = (int32_t)grid_size[2];
+    for (int a = 0; a < 3; ++a) { p.voxel_min[a] = (float)voxel_min[a]; p.voxel_size[a] = (float)voxel_size[a]; }
+    p.epsilon = epsilon;
+    p.channels = 1; p.depth_bins = 2;
+    p.proj_stride = (int32_t)(projection_matrices.size(2) * 4);
+    TORCH_CHECK(p.grid_x > 0 && p.grid_y > 0 && p.grid_z > 0, "flashbevpool_ext: grid_size must be positive");
+    auto dev = projection_matrices.device();
+    std::vector<int64_t> shp = {p.batch, p.grid_y, p.grid_x, p.num_cams, p.grid_z};
+    at::Tensor mask = at::empty(shp, at::TensorOptions().device(dev).dtype(at::kByte));
+    shp.push_back(4);
+    at::Tensor idx = at::empty(shp, at::TensorOptions().device(dev).dtype(at::kInt));
+    shp.back() = 2;
+    at::Tensor frac = at::empty(shp, at::TensorOptions().device(dev).dtype(at::kFloat));
+    DeviceScope scope(projection_matrices.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(projection_matrices.get_device()).stream();
+    raise_on(fbev_sample_geometry(&p, projection_matrices.data_ptr<float>(), mask.data_ptr<uint8_t>(),
+                                  idx.data_ptr<int32_t>(), frac.data_ptr<float>(), st),
+             "fbev_sample_geometry");
+    return {mask, idx, frac};
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    namespace py = pybind11;
+    m.def("flash_bevpool_forward", &flash_bevpool_forward, "fused camera->BEV pooling, forward",
+          py::arg("depth_params"), py::arg("image_feats"), py::arg("projection_matrices"), py::arg("feature_size"),
+          py::arg("image_size"), py::arg("grid_size"), py::arg("voxel_size_x"), py::arg("voxel_size_y"),
+          py::arg("voxel_size_z"), py::arg("voxel_x_min"), py::arg("voxel_y_min"), py::arg("voxel_z_min"),
+          py::arg("out"), py::arg("total_threads"), py::arg("depth_distribution"), py::arg("use_shared_memory"),
+          py::arg("optimize_z_precompute"), py::arg("use_warp_kernel"), py::arg("use_vectorized_load"),
+          py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f, py::arg("depth_min") = 1.0f,
+          py::arg("depth_step") = 1.0f, py::arg("reduction") = 0);
+    m.def("flash_bevpool_backward", &flash_bevpool_backward, "fused camera->BEV pooling, backward",
+          py::arg("out_grad"), py::arg("depth_params"), py::arg("image_feats"), py::arg("projection_matrices"),
+          py::arg("feature_size"), py::arg("image_size"), py::arg("roi_range"), py::arg("grid_size"),
+          py::arg("depth_params_grad"), py::arg("image_feats_grad"), py::arg("total_threads"),
+          py::arg("depth_distribution"), py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f,
+          py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0);
+    m.def("sample_geometry", &sample_geometry, "per-sample validity mask and corner indices (parity hook)",
+          py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
+          py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);
+    m.def("abi_version", []() { return fbev_abi_version(); });
+}

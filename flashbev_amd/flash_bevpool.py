@@ -1,0 +1,170 @@
+"""Python-facing operator of the fused camera->BEV pooling, with the reference's names,
+argument order and defaults (flashbev/flashbevpool/flash_bevpool.py:11-178):
+
+    FlashBEVPool.apply(depth_params, image_feats, projection_matrices, feature_size,
+                       image_size, roi_range, grid_size, depth_distribution=0, ...)
+    flash_bevpool(image_feats, depth_params, projection_matrices, ...)   # feats first
+
+Differences from the reference, all additive:
+  * float16 / bfloat16 features and depth are consumed as they are (fp32 accumulation, fp32
+    result and fp32 gradient buffers); the reference up-casts copies
+    (flash_bevpool.py:47-49).
+  * ``projection_matrices`` may be [B,N,3,4] or [B,N,4,4].
+  * ``image_size``, ``roi_range`` and ``grid_size`` may be CPU tensors or plain sequences;
+    then the call never synchronises with the device (the reference does six ``.item()``
+    reads per call, flash_bevpool.py:58-67).
+  * ``depth_distribution=2`` selects a categorical depth model over ``depth_range=(d_min,
+    d_step)`` bins; ``reduction="sum"`` skips the division by the valid-sample count.
+  * the backward pass returns the true gradient with respect to the depth parameters (the
+    reference kernel's expression, flash_bevpool_cuda.cu:665-674, is not a derivative).
+The four kernel-variant switches (use_shared_memory, optimize_z_precompute,
+use_warp_kernel, use_vectorized_load) are accepted and select nothing: they never change
+results in the reference either.
+"""
+from __future__ import annotations
+
+import weakref
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from ._native import load_ext
+
+_SUPPORTED = (torch.float32, torch.float16, torch.bfloat16)
+_host_cache: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()
+
+
+def _host_values(x, n: int, name: str):
+    """Values of a small size/range argument as Python numbers.
+
+    Sequences and CPU tensors cost nothing.  A device tensor costs one synchronous copy,
+    remembered per tensor object and version so that a tensor reused across calls (a
+    registered buffer, say) is read once.
+    """
+    if isinstance(x, torch.Tensor):
+        if x.numel() != n:
+            raise ValueError(f"{name} must have {n} elements, got shape {tuple(x.shape)}")
+        if x.device.type == "cpu":
+            return x.reshape(-1).tolist()
+        hit = _host_cache.get(x)
+        if hit is not None and hit[0] == x._version:
+            return hit[1]
+        vals = x.detach().reshape(-1).tolist()
+        _host_cache[x] = (x._version, vals)
+        return vals
+    vals = list(x)
+    if len(vals) != n:
+        raise ValueError(f"{name} must have {n} elements, got {len(vals)}")
+    return vals
+
+
+def voxel_geometry(roi_range: Sequence[float], grid_size: Sequence[int]):
+    """(voxel_min[3], voxel_size[3]) as fp32 values: size = (max - min) / grid, one rounded
+    fp32 subtraction and one rounded fp32 division (flash_bevpool.py:62-67)."""
+    r = np.asarray(roi_range, dtype=np.float32)
+    g = np.asarray(grid_size, dtype=np.float32)
+    size = (r[1::2] - r[0::2]) / g
+    return [float(v) for v in r[0::2]], [float(v) for v in size]
+
+
+class FlashBEVPool(torch.autograd.Function):
+    """Fused projection + depth weighting + bilinear sampling + reduction over cameras and
+    height bins.  Returns BEV features [B, Y, X, C] in float32."""
+
+    @staticmethod
+    def forward(ctx, depth_params, image_feats, projection_matrices, feature_size, image_size,
+                roi_range, grid_size, depth_distribution=0, use_shared_memory=True,
+                optimize_z_precompute=True, use_warp_kernel=False, use_vectorized_load=False,
+                epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=None, reduction="mean"):
+        ext = load_ext()
+        if not (isinstance(image_feats, torch.Tensor) and image_feats.is_cuda):
+            raise RuntimeError("flash_bevpool: image_feats must be a tensor on a ROCm GPU; "
+                               "this operator has no CPU path")
+        if depth_params.dtype != image_feats.dtype or image_feats.dtype not in _SUPPORTED:
+            depth_params = depth_params.float()
+            image_feats = image_feats.float()
+        depth_params = depth_params.contiguous()
+        image_feats = image_feats.contiguous()
+        projection_matrices = projection_matrices.contiguous().float()
+        if reduction not in ("mean", "sum"):
+            raise ValueError(f"reduction must be 'mean' or 'sum', got {reduction!r}")
+        depth_distribution = int(depth_distribution)
+        if depth_distribution not in (0, 1, 2):
+            raise ValueError(f"depth_distribution must be 0 (gaussian), 1 (laplace) or 2 "
+                             f"(categorical), got {depth_distribution}")
+        if depth_distribution == 2 and depth_range is None:
+            raise ValueError("depth_distribution=2 needs depth_range=(d_min, d_step)")
+        d_min, d_step = (1.0, 1.0) if depth_range is None else (float(depth_range[0]), float(depth_range[1]))
+
+        B, N, H, W, C = image_feats.shape
+        grid = [int(v) for v in _host_values(grid_size, 3, "grid_size")]
+        image = [int(v) for v in _host_values(image_size, 2, "image_size")]
+        roi = [float(v) for v in _host_values(roi_range, 6, "roi_range")]
+        vmin, vsize = voxel_geometry(roi, grid)
+
+        # feature_size repeats the feature tensor's (H, W) per camera; hand the extension a
+        # host copy built from the shape unless the caller already gave a host tensor.
+        if isinstance(feature_size, torch.Tensor) and feature_size.device.type == "cpu":
+            fs_host = feature_size.to(torch.int32).contiguous()
+        else:
+            fs_host = torch.tensor([H, W], dtype=torch.int32).repeat(B * N)
+        image_t = torch.tensor(image, dtype=torch.int32)
+        grid_t = torch.tensor(grid, dtype=torch.int32)
+        roi_t = torch.tensor(roi, dtype=torch.float32)
+
+        out = torch.empty((B, grid[1], grid[0], C), dtype=torch.float32, device=image_feats.device)
+        red = 0 if reduction == "mean" else 1
+        ext.flash_bevpool_forward(
+            depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
+            vsize[0], vsize[1], vsize[2], vmin[0], vmin[1], vmin[2], out, out.numel(),
+            depth_distribution, bool(use_shared_memory), bool(optimize_z_precompute),
+            bool(use_warp_kernel), bool(use_vectorized_load), float(epsilon),
+            float(depth_weight_threshold), d_min, d_step, red)
+
+        ctx.save_for_backward(depth_params, image_feats, projection_matrices)
+        ctx.host = (fs_host, image_t, roi_t, grid_t)
+        ctx.total_threads = out.numel()
+        ctx.depth_distribution = depth_distribution
+        ctx.epsilon = float(epsilon)
+        ctx.depth_weight_threshold = float(depth_weight_threshold)
+        ctx.depth_range = (d_min, d_step)
+        ctx.reduction = red
+        return out
+
+    @staticmethod
+    def backward(ctx, out_grad):
+        ext = load_ext()
+        depth_params, image_feats, projection_matrices = ctx.saved_tensors
+        fs_host, image_t, roi_t, grid_t = ctx.host
+        need_depth, need_feats = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        depth_params_grad = torch.zeros(depth_params.shape, dtype=torch.float32,
+                                        device=depth_params.device) if need_depth else None
+        image_feats_grad = torch.zeros(image_feats.shape, dtype=torch.float32,
+                                       device=image_feats.device) if need_feats else None
+        if need_depth or need_feats:
+            ext.flash_bevpool_backward(
+                out_grad.contiguous().float(), depth_params, image_feats, projection_matrices,
+                fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
+                ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
+                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction)
+        return (depth_params_grad, image_feats_grad) + (None,) * 14
+
+
+def flash_bevpool(image_feats, depth_params, projection_matrices, feature_size, image_size,
+                  roi_range, grid_size, depth_distribution=0, use_shared_memory=True,
+                  optimize_z_precompute=True, use_warp_kernel=False, use_vectorized_load=False,
+                  epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=None, reduction="mean"):
+    """Keyword-friendly wrapper; note ``image_feats`` comes first here and second in
+    ``FlashBEVPool.apply`` (as in flashbev/flashbevpool/flash_bevpool.py:139-178).
+
+    image_feats [B,N,H,W,C], depth_params [B,N,H,W,2] (mean, sigma) or [B,N,H,W,D] for the
+    categorical model, projection_matrices [B,N,3|4,4], feature_size [B,N,2], image_size
+    [2] (rows, cols), roi_range [6] (xmin,xmax,ymin,ymax,zmin,zmax), grid_size [3]
+    (x,y,z).  Returns [B, Y, X, C] float32.
+    """
+    return FlashBEVPool.apply(depth_params, image_feats, projection_matrices, feature_size,
+                              image_size, roi_range, grid_size, depth_distribution,
+                              use_shared_memory, optimize_z_precompute, use_warp_kernel,
+                              use_vectorized_load, epsilon, depth_weight_threshold, depth_range,
+                              reduction)

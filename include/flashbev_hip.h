@@ -1,0 +1,119 @@
+/*
+ * flashbev_hip.h -- C ABI of libflashbev_hip.so: fused camera->BEV pooling for gfx950.
+ *
+ * Plain pointers and sizes only; no torch types.  All data pointers are DEVICE pointers
+ * valid on the device that is current when the call is made; `stream` is a hipStream_t
+ * passed as void* (NULL = the null stream).  Every call is asynchronous with respect to
+ * the host and allocates nothing.  Return value: FBEV_OK or a negative fbev_status.
+ *
+ * Tensor layouts (all dense, row-major, innermost index last):
+ *   feats  [B, N, H, W, C]   fp32 / fp16 / bf16 (in_dtype), channels last
+ *   depth  [B, N, H, W, Dd]  same dtype as feats; Dd = 2 (mean, sigma) for the Gaussian /
+ *                            Laplace models, Dd = depth_bins for the categorical model
+ *   proj   [B, N, proj_stride] fp32; the first 12 floats of each block are a row-major
+ *                            3x4 projection matrix (proj_stride = 12 for [B,N,3,4],
+ *                            16 for [B,N,4,4])
+ *   out / grad_out [B, grid_y, grid_x, C] fp32
+ *   d_feats [B, N, H, W, C] fp32,  d_depth [B, N, H, W, Dd] fp32
+ */
+#ifndef FLASHBEV_HIP_H
+#define FLASHBEV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FBEV_ABI_VERSION 1
+
+typedef enum fbev_status {
+    FBEV_OK = 0,
+    FBEV_ERR_NULL = -1,        /* a required pointer is NULL */
+    FBEV_ERR_SHAPE = -2,       /* a size is <= 0 or inconsistent */
+    FBEV_ERR_UNSUPPORTED = -3, /* unknown dtype / depth model / reduction */
+    FBEV_ERR_TOO_LARGE = -4,   /* an element count does not fit the 32-bit indices used */
+    FBEV_ERR_ALIGNMENT = -5,   /* a pointer is not aligned to its element type */
+    FBEV_ERR_LAUNCH = -6       /* the HIP runtime reported a launch error */
+} fbev_status;
+
+enum { FBEV_F32 = 0, FBEV_F16 = 1, FBEV_BF16 = 2 };
+enum { FBEV_GAUSSIAN = 0, FBEV_LAPLACE = 1, FBEV_CATEGORICAL = 2 };
+enum { FBEV_REDUCE_MEAN = 0, FBEV_REDUCE_SUM = 1 };
+
+/*
+ * Problem description.  It gathers, by value, what the reference passes as scalars and
+ * small tensors to flash_bevpool_forward / flash_bevpool_backward
+ * (flashbev/flashbevpool/src/flash_bevpool.cpp:79-101,168-183).
+ */
+typedef struct fbev_problem {
+    int32_t batch;       /* B */
+    int32_t num_cams;    /* N */
+    int32_t feat_h;      /* H: rows of every camera's feature map */
+    int32_t feat_w;      /* W */
+    int32_t channels;    /* C */
+    int32_t image_h;     /* Hi: image rows the projection matrices refer to */
+    int32_t image_w;     /* Wi */
+    int32_t grid_x;      /* BEV cells along x */
+    int32_t grid_y;
+    int32_t grid_z;      /* height bins reduced per cell */
+    float voxel_min[3];  /* lower edge of the region of interest along x, y, z */
+    float voxel_size[3]; /* cell size along x, y, z: (max - min) / grid, an fp32 division;
+                            cell i has its centre at min + (i + 0.5) * size */
+    float epsilon;       /* added to sigma; lower clamp of the perspective divisor */
+    float depth_weight_threshold; /* samples with weight < threshold are dropped */
+    int32_t depth_distribution;   /* FBEV_GAUSSIAN / FBEV_LAPLACE / FBEV_CATEGORICAL */
+    int32_t depth_bins;  /* Dd: 2 for the parametric models */
+    float depth_min;     /* categorical: depth of bin 0 */
+    float depth_step;    /* categorical: spacing of the bins */
+    int32_t in_dtype;    /* FBEV_F32 / FBEV_F16 / FBEV_BF16 for feats and depth */
+    int32_t reduction;   /* FBEV_REDUCE_MEAN (the reference's) / FBEV_REDUCE_SUM */
+    int32_t proj_stride; /* 12 or 16 */
+} fbev_problem;
+
+/*
+ * Forward: out[b,y,x,:] = mean (or sum) over the valid (camera, height-bin) samples of
+ * depth_weight * bilinear(feats).  Every element of `out` is written (cells that no
+ * camera sees get 0), so `out` need not be zeroed.
+ * Replaces the launcher flash_bevpool(...) (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:757-865)
+ * as bound by flash_bevpool_forward (flashbev/flashbevpool/src/flash_bevpool.cpp:79-166).
+ */
+int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, const float *proj,
+                 float *out, void *stream);
+
+/*
+ * Backward: ACCUMULATES the exact gradients of fbev_forward into d_depth and d_feats, which
+ * the caller zero-fills (the reference's ownership rule, flashbev/flashbevpool/flash_bevpool.py:115-116).
+ * Either gradient pointer may be NULL to skip that gradient.
+ * Replaces flash_bevpool_grad(...) (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:867-937) as bound by
+ * flash_bevpool_backward (flashbev/flashbevpool/src/flash_bevpool.cpp:168-241).  The depth gradient is
+ * the true derivative of the forward, not the reference kernel's expression at
+ * flash_bevpool_cuda.cu:665-674.
+ */
+int fbev_backward(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                  const float *proj, float *d_depth, float *d_feats, void *stream);
+
+/*
+ * Inspection hook for parity tests: per (b, y, x, camera, height-bin) sample, in that
+ * order, the projection validity and the bilinear corner indices the kernels use.
+ *   mask  uint8  [B,gy,gx,N,gz]      1 = depth > 0 and inside the feature map
+ *   idx   int32  [B,gy,gx,N,gz,4]    (u0,u1,v0,v1), -1 where mask is 0
+ *   frac  float  [B,gy,gx,N,gz,2]    (du,dv), 0 where mask is 0
+ * Any of the three may be NULL.  p->channels, in_dtype and the depth fields are ignored.
+ * Restates flashbev/flashbevpool/src/flash_bevpool_cuda.cu:102-159; the reference exports no such call.
+ */
+int fbev_sample_geometry(const fbev_problem *p, const float *proj, uint8_t *mask, int32_t *idx,
+                         float *frac, void *stream);
+
+/* Compulsory bytes moved by one call: every operand tensor once (backward != 0 selects the backward). */
+uint64_t fbev_algorithmic_bytes(const fbev_problem *p, int backward);
+
+const char *fbev_status_string(int status);
+int fbev_abi_version(void);
+size_t fbev_problem_size(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHBEV_HIP_H */

@@ -1,0 +1,103 @@
+"""Shared helpers of the test suite: oracle calls on a workload, error metrics."""
+import numpy as np
+import torch
+
+from flashbev_amd import capi
+from flashbev_amd.flash_bevpool import voxel_geometry
+from oracle import c_oracle, dense_torch
+
+RTOL, ATOL = 1e-4, 1e-5   # fp32 outputs and gradients (the stated parity tolerance)
+
+
+def op_kwargs(w, dist, thr=1e-6, eps=1e-6):
+    return dict(image_size=w.image_hw, roi_range=w.roi_range, grid_size=w.grid_size,
+                depth_distribution=dist, epsilon=eps, depth_weight_threshold=thr,
+                depth_range=w.depth_range)
+
+
+def oracle_forward(x, w, dist, thr=1e-6, eps=1e-6, **extra):
+    return c_oracle.forward(x["depth_params"].float().cpu().numpy(), x["image_feats"].float().cpu().numpy(),
+                            x["projection_matrices"].cpu().numpy(), **op_kwargs(w, dist, thr, eps), **extra)
+
+
+def oracle_backward(x, w, dist, thr=1e-6, eps=1e-6, **extra):
+    return c_oracle.backward(x["grad_out"].cpu().numpy(), x["depth_params"].float().cpu().numpy(),
+                             x["image_feats"].float().cpu().numpy(), x["projection_matrices"].cpu().numpy(),
+                             **op_kwargs(w, dist, thr, eps), **extra)
+
+
+def violations(got, want, rtol=RTOL, atol=ATOL):
+    """(count of elements outside |got-want| <= atol + rtol*|want|, max |diff|, max diff/tol)."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    d = np.abs(got - want)
+    tol = atol + rtol * np.abs(want)
+    bad = ~(d <= tol)          # NaN counts as a violation
+    return int(bad.sum()), float(np.nanmax(d)) if d.size else 0.0, float(np.nanmax(d / tol)) if d.size else 0.0
+
+
+def reference_metrics(got, want):
+    """The statistics of the reference's difference harness (tools/profile_differences.py:17-67)."""
+    a = torch.as_tensor(np.asarray(got), dtype=torch.float64).flatten()
+    b = torch.as_tensor(np.asarray(want), dtype=torch.float64).flatten()
+    diff = a - b
+    rel = diff.abs() / b.abs().clamp(min=1e-8)
+    cos = torch.nn.functional.cosine_similarity(a.unsqueeze(0), b.unsqueeze(0)).item()
+    return {"mse": (diff ** 2).mean().item(), "mae": diff.abs().mean().item(),
+            "max_abs": diff.abs().max().item(), "mean_rel": rel.mean().item(), "cosine": cos}
+
+
+def dtype_code(t):
+    return {torch.float32: capi.FBEV_F32, torch.float16: capi.FBEV_F16, torch.bfloat16: capi.FBEV_BF16}[t]
+
+
+def problem_for(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN):
+    """fbev_problem of a workload's tensors (device or host)."""
+    B, N, H, W, C = x["image_feats"].shape
+    vmin, vsize = voxel_geometry(w.roi_range, w.grid_size)
+    return capi.make_problem(B, N, (H, W), C, w.image_hw, w.grid_size, vmin, vsize, depth_distribution=dist,
+                             depth_bins=x["depth_params"].shape[-1], epsilon=eps, depth_weight_threshold=thr,
+                             depth_range=w.depth_range, in_dtype=dtype_code(x["image_feats"].dtype),
+                             reduction=reduction, proj_stride=x["projection_matrices"].shape[-2] * 4)
+
+
+def capi_forward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN):
+    """Forward through the C ABI on the tensors' device; returns out [B,gy,gx,C] float32."""
+    p = problem_for(x, w, dist, thr, eps, reduction)
+    out = torch.full((p.batch, p.grid_y, p.grid_x, p.channels), float("nan"), dtype=torch.float32,
+                     device=x["image_feats"].device)
+    st = torch.cuda.current_stream().cuda_stream
+    capi.check(capi.forward(p, x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
+                            x["projection_matrices"].data_ptr(), out.data_ptr(), st), "fbev_forward")
+    torch.cuda.synchronize()
+    return out
+
+
+def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, want=(True, True)):
+    p = problem_for(x, w, dist, thr, eps, reduction)
+    dev = x["image_feats"].device
+    dd = torch.zeros(x["depth_params"].shape, dtype=torch.float32, device=dev) if want[0] else None
+    df = torch.zeros(x["image_feats"].shape, dtype=torch.float32, device=dev) if want[1] else None
+    st = torch.cuda.current_stream().cuda_stream
+    capi.check(capi.backward(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
+                             x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(),
+                             dd.data_ptr() if dd is not None else None,
+                             df.data_ptr() if df is not None else None, st), "fbev_backward")
+    torch.cuda.synchronize()
+    return dd, df
+
+
+def capi_geometry(proj, w):
+    B, N = proj.shape[:2]
+    vmin, vsize = voxel_geometry(w.roi_range, w.grid_size)
+    p = capi.make_problem(B, N, w.feat_hw, 1, w.image_hw, w.grid_size, vmin, vsize,
+                          proj_stride=proj.shape[-2] * 4)
+    gx, gy, gz = w.grid_size
+    shp = (B, gy, gx, N, gz)
+    mask = torch.empty(shp, dtype=torch.uint8, device=proj.device)
+    idx = torch.empty(shp + (4,), dtype=torch.int32, device=proj.device)
+    frac = torch.empty(shp + (2,), dtype=torch.float32, device=proj.device)
+    capi.check(capi.sample_geometry(p, proj.data_ptr(), mask.data_ptr(), idx.data_ptr(), frac.data_ptr(),
+                                    torch.cuda.current_stream().cuda_stream), "fbev_sample_geometry")
+    torch.cuda.synchronize()
+    return mask, idx, frac
