@@ -43,8 +43,9 @@ DIST_OF = {"gaussian": (0, "parametric"), "laplace": (1, "parametric"), "categor
 class Runner:
     """Pre-allocated buffers and the four queued operations of one step."""
 
-    def __init__(self, w, depth_name: str, device: str = "cuda:0"):
+    def __init__(self, w, depth_name: str, device: str = "cuda:0", backward_mode: int = 0):
         self.w = w
+        self.backward_mode = backward_mode
         self.dist, self.model = DIST_OF[depth_name]
         self.ext = load_ext()
         x = make_inputs(w, self.model, device=device, with_grad_out=True)
@@ -74,7 +75,7 @@ class Runner:
         self.ext.flash_bevpool_backward(
             x["grad_out"], x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
             x["image_size"], x["roi_range"], x["grid_size"], self.d_depth, self.d_feats, self.out.numel(),
-            self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0)
+            self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0, self.backward_mode, -1)
 
 
 def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):

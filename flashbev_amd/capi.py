@@ -15,7 +15,8 @@ FBEV_F32, FBEV_F16, FBEV_BF16 = 0, 1, 2
 FBEV_GAUSSIAN, FBEV_LAPLACE, FBEV_CATEGORICAL = 0, 1, 2
 FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
-EXPORTS = ("fbev_forward", "fbev_backward", "fbev_sample_geometry", "fbev_algorithmic_bytes",
+EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_max_pairs",
+           "fbev_backward_workspace_bytes", "fbev_sample_geometry", "fbev_algorithmic_bytes",
            "fbev_status_string", "fbev_abi_version", "fbev_problem_size")
 
 
@@ -45,6 +46,12 @@ def load() -> ctypes.CDLL:
         lib.fbev_forward.restype = ctypes.c_int
         lib.fbev_backward.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp]
         lib.fbev_backward.restype = ctypes.c_int
+        lib.fbev_backward_gather.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp]
+        lib.fbev_backward_gather.restype = ctypes.c_int
+        lib.fbev_backward_max_pairs.argtypes = [pp]
+        lib.fbev_backward_max_pairs.restype = ctypes.c_uint64
+        lib.fbev_backward_workspace_bytes.argtypes = [pp, ctypes.c_uint64]
+        lib.fbev_backward_workspace_bytes.restype = ctypes.c_size_t
         lib.fbev_sample_geometry.argtypes = [pp, vp, vp, vp, vp, vp]
         lib.fbev_sample_geometry.restype = ctypes.c_int
         lib.fbev_algorithmic_bytes.argtypes = [pp, ctypes.c_int]
@@ -106,6 +113,22 @@ def backward(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, 
              d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], stream: int = 0) -> int:
     return load().fbev_backward(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
                                 _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), _p(stream))
+
+
+def backward_gather(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
+                    d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], workspace_ptr: int,
+                    workspace_bytes: int, stream: int = 0) -> int:
+    return load().fbev_backward_gather(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
+                                       _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), _p(workspace_ptr),
+                                       ctypes.c_size_t(int(workspace_bytes)), _p(stream))
+
+
+def backward_max_pairs(p: FbevProblem) -> int:
+    return int(load().fbev_backward_max_pairs(ctypes.byref(p)))
+
+
+def backward_workspace_bytes(p: FbevProblem, pair_capacity: int) -> int:
+    return int(load().fbev_backward_workspace_bytes(ctypes.byref(p), ctypes.c_uint64(int(pair_capacity))))
 
 
 def sample_geometry(p: FbevProblem, proj_ptr: int, mask_ptr: Optional[int], idx_ptr: Optional[int],

@@ -232,9 +232,15 @@ __device__ __forceinline__ unsigned long long lanemask_lt(int lane) {
 //           backward: raw bilinear corner weights (w00, w01, w10, w11)
 //   word 1: four texel indices ((b*N+n)*H + v)*W + u as int bits (t00, t01, t10, t11)
 //   word 2 (backward only): wgt, a, b, (k0 | k1 << 16)
-template <int ENTRY_F4, typename T, bool BACKWARD>
+//   word 3 (backward through the inverse map only): for each corner the position of its
+//           (cell, coefficient) pair in the texel-sorted pair array, or -1 if the array is full
+enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2 };
+
+template <int ENTRY_F4, typename T, int MODE>
 __device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const T *__restrict__ depth,
-                                        int b, int q0, int lane, float4 *lst, volatile int *cnt) {
+                                        int b, int q0, int lane, float4 *lst, volatile int *cnt,
+                                        int *__restrict__ cursor = nullptr, int pair_cap = 0) {
+    constexpr bool BACKWARD = MODE != kModeForward;
     const int total = k.slots * k.NZ;
     for (int base = 0; base < total; base += kWave) {
         int idx = base + lane;
@@ -286,6 +292,20 @@ __device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const
             e[1] = make_float4(__int_as_float(tx.x), __int_as_float(tx.y), __int_as_float(tx.z),
                                __int_as_float(tx.w));
             if (ENTRY_F4 > 2) e[2] = w2;
+            if (MODE == kModeFill) {
+                // claim one slot per corner in the texel's segment of the pair array; the four
+                // requests of all lanes are in flight together, so the round trip is paid once
+                int p0 = atomicAdd(cursor + tx.x, 1);
+                int p1 = atomicAdd(cursor + tx.y, 1);
+                int p2 = atomicAdd(cursor + tx.z, 1);
+                int p3 = atomicAdd(cursor + tx.w, 1);
+                p0 = p0 < pair_cap ? p0 : -1;
+                p1 = p1 < pair_cap ? p1 : -1;
+                p2 = p2 < pair_cap ? p2 : -1;
+                p3 = p3 < pair_cap ? p3 : -1;
+                e[ENTRY_F4 - 1] = make_float4(__int_as_float(p0), __int_as_float(p1), __int_as_float(p2),
+                                              __int_as_float(p3));
+            }
         }
         if (active && lane == lo) cnt[slot] = old + __popcll(m & seg);
     }
@@ -325,7 +345,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
         const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
         if (lane < 16) cnt[lane] = 0;
-        phase_a<2, T, false>(k, Pm, depth, b, q0, lane, lst, cnt);
+        phase_a<2, T, kModeForward>(k, Pm, depth, b, q0, lane, lst, cnt);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
@@ -395,13 +415,100 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
 }
 
 // ---------------------------------------------------------------- backward
+// Two ways to form the feature gradient, which is a sum over all samples that touch a texel:
+//   scatter      fbev_backward_cells_kernel<.., false>: one hardware fp32 atomic per (sample,
+//                corner, channel).  Needs no workspace; slow under contention.
+//   inverse map  count the samples per texel, prefix-sum the counts, let the cell pass
+//                (fbev_backward_cells_kernel<.., true>) drop one 16-byte (cell, coefficient)
+//                pair per sample corner into the texel's segment, then gather per texel
+//                (fbev_backward_texel_kernel): the same coalesced row reads as the forward
+//                pass, no floating-point atomics, each gradient row written once.
 __device__ __forceinline__ void atomic_add_f32(float *p, float v) { unsafeAtomicAdd(p, v); }
 
-template <typename T, int VEC, int CPL>
-__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_kernel(
+struct Pair {      // 16 bytes
+    int cell;      // row of grad_out: (b * gy + iy) * gx + ix
+    float coef;    // d out[cell, c] / d feats[texel, c]
+    float da, db;  // this sample's contribution to d_depth[texel, 0] and [texel, 1] (parametric models)
+};
+
+__global__ __launch_bounds__(256) void fbev_fill_zero_kernel(int *p, long long n) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// One thread per (cell, camera, height) sample: count, per texel, the sample corners that
+// will contribute.  Runs exactly the decisions of phase A (same functions, same inputs).
+template <typename T>
+__global__ __launch_bounds__(256) void fbev_count_kernel(KParams k, const T *__restrict__ depth,
+                                                         const float *__restrict__ proj, int *__restrict__ counts,
+                                                         long long total) {
+    long long s = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (s >= total) return;
+    int iz = (int)(s % k.gz);
+    long long r = s / k.gz;
+    int n = (int)(r % k.N); r /= k.N;
+    int ix = (int)(r % k.gx); r /= k.gx;
+    int iy = (int)(r % k.gy);
+    int b = (int)(r / k.gy);
+    const float *P = proj + (size_t)(b * k.N + n) * k.proj_stride;
+    float Pl[12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) Pl[i] = P[i];
+    Geom g = project_sample(k, Pl, voxel_coord(k.xmin, ix, k.vx), voxel_coord(k.ymin, iy, k.vy),
+                            voxel_coord(k.zmin, iz, k.vz));
+    if (!g.valid) return;
+    float w00 = (1.0f - g.du) * (1.0f - g.dv);
+    float w01 = (1.0f - g.du) * g.dv;
+    float w10 = g.du * (1.0f - g.dv);
+    float w11 = g.du * g.dv;
+    int rowbase = (b * k.N + n) * k.H;
+    int t00 = (rowbase + g.v0) * k.W + g.u0;
+    int t01 = (rowbase + g.v1) * k.W + g.u0;
+    int t10 = (rowbase + g.v0) * k.W + g.u1;
+    int t11 = (rowbase + g.v1) * k.W + g.u1;
+    DepthEval e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
+    if (!e.keep) return;
+    atomicAdd(counts + t00, 1);
+    atomicAdd(counts + t01, 1);
+    atomicAdd(counts + t10, 1);
+    atomicAdd(counts + t11, 1);
+}
+
+// In-place exclusive prefix sum of v[0..n) by one block; v[n] receives the total.
+__global__ __launch_bounds__(1024) void fbev_scan_kernel(int *v, int n) {
+    __shared__ int part[1024];
+    const int tid = threadIdx.x;
+    const int chunk = (n + 1023) / 1024;
+    const int lo = min(tid * chunk, n), hi = min(lo + chunk, n);
+    int sum = 0;
+    for (int i = lo; i < hi; ++i) sum += v[i];
+    part[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        int add = tid >= off ? part[tid - off] : 0;
+        __syncthreads();
+        part[tid] += add;
+        __syncthreads();
+    }
+    int run = part[tid] - sum;
+    for (int i = lo; i < hi; ++i) {
+        int c = v[i];
+        v[i] = run;
+        run += c;
+    }
+    if (tid == 1023) v[n] = part[1023];
+}
+
+// Cell pass of the backward.  FILL = false: scatter with atomics.  FILL = true: write pairs.
+// `cursor` holds, on entry, the start of every texel's segment; phase A advances it, so on
+// exit cursor[t] is the END of texel t's segment (= the start of texel t+1's).
+template <typename T, int VEC, int CPL, bool FILL>
+__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_kernel(
     KParams k, const float *__restrict__ grad_out, const T *__restrict__ depth, const T *__restrict__ feats,
-    const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats) {
+    const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
+    int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap) {
     extern __shared__ float4 smem[];
+    constexpr int EF4 = FILL ? 4 : 3;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
@@ -410,7 +517,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_kernel(
 
     float *Pm = reinterpret_cast<float *>(smem);
     const int p_f4 = (k.N * 12 + 3) / 4;
-    const int per_wave_f4 = 4 + k.slots * k.list_cap * 3;
+    const int per_wave_f4 = 4 + k.slots * k.list_cap * EF4;
     float4 *wbase = smem + p_f4 + wave * per_wave_f4;
     volatile int *cnt = reinterpret_cast<volatile int *>(wbase);
     float4 *lst = wbase + 4;
@@ -425,12 +532,15 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_kernel(
     const bool carrier = slot < k.slots;
     const int span = k.lanes_per_slot * VEC * CPL;
     const int Dd = k.Dd;
+    const bool parametric = k.dist != FBEV_CATEGORICAL;
+    // the inner product <grad_out, sampled feature> is only needed for the depth gradient
+    const bool need_G = d_depth != nullptr;
 
     for (int r = 0; r < k.rounds; ++r) {
         const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
         if (lane < 16) cnt[lane] = 0;
-        phase_a<3, T, true>(k, Pm, depth, b, q0, lane, lst, cnt);
+        phase_a<EF4, T, FILL ? kModeFill : kModeScatter>(k, Pm, depth, b, q0, lane, lst, cnt, cursor, pair_cap);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
@@ -442,11 +552,13 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_kernel(
         int n_max = n;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) n_max = max(n_max, __shfl_xor(n_max, off, kWave));
-        const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * 3;
-        const float *go = grad_out + (((size_t)b * k.gy + iy) * k.gx + ix) * k.C;
+        const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * EF4;
+        const int cell = (b * k.gy + iy) * k.gx + ix;
+        const float *go = grad_out + (size_t)cell * k.C;
         const float inv = (k.reduce_sum || n == 0) ? 1.0f : 1.0f / (float)n;
 
         for (int c0 = 0; c0 < k.C; c0 += span) {
+            const bool first_pass = c0 == 0;
             float g[CPL][VEC];
 #pragma unroll
             for (int j = 0; j < CPL; ++j) {
@@ -469,21 +581,25 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_kernel(
             for (int e = 0; e < n_max; ++e) {
                 const bool live = e < n;
                 float G = 0.0f;
-                float4 w = make_float4(0.f, 0.f, 0.f, 0.f), tf = w, dw = w;
+                float4 w = make_float4(0.f, 0.f, 0.f, 0.f), tf = w, dw = w, pf = w;
                 if (live) {
-                    w = my[3 * e];
-                    tf = my[3 * e + 1];
-                    dw = my[3 * e + 2];
+                    w = my[EF4 * e];
+                    tf = my[EF4 * e + 1];
+                    dw = my[EF4 * e + 2];
+                    if (FILL) pf = my[EF4 * e + 3];
                     const size_t o00 = (size_t)__float_as_int(tf.x) * k.C;
                     const size_t o01 = (size_t)__float_as_int(tf.y) * k.C;
                     const size_t o10 = (size_t)__float_as_int(tf.z) * k.C;
                     const size_t o11 = (size_t)__float_as_int(tf.w) * k.C;
                     const float a00 = w.x * dw.x, a01 = w.y * dw.x, a10 = w.z * dw.x, a11 = w.w * dw.x;
+                    // corners whose pair found no room in the pair array fall back to atomics
+                    const bool s00 = !FILL || __float_as_int(pf.x) < 0, s01 = !FILL || __float_as_int(pf.y) < 0;
+                    const bool s10 = !FILL || __float_as_int(pf.z) < 0, s11 = !FILL || __float_as_int(pf.w) < 0;
 #pragma unroll
                     for (int j = 0; j < CPL; ++j) {
                         int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
                         if (ch < k.C) {
-                            if (d_depth != nullptr) {
+                            if (need_G) {
                                 float f00[VEC], f01[VEC], f10[VEC], f11[VEC];
                                 VecLoad<T, VEC>::ld(feats + o00 + ch, f00);
                                 VecLoad<T, VEC>::ld(feats + o01 + ch, f01);
@@ -498,41 +614,134 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_kernel(
                             if (d_feats != nullptr) {
 #pragma unroll
                                 for (int v = 0; v < VEC; ++v) {
-                                    atomic_add_f32(d_feats + o00 + ch + v, g[j][v] * a00);
-                                    atomic_add_f32(d_feats + o01 + ch + v, g[j][v] * a01);
-                                    atomic_add_f32(d_feats + o10 + ch + v, g[j][v] * a10);
-                                    atomic_add_f32(d_feats + o11 + ch + v, g[j][v] * a11);
+                                    if (s00) atomic_add_f32(d_feats + o00 + ch + v, g[j][v] * a00);
+                                    if (s01) atomic_add_f32(d_feats + o01 + ch + v, g[j][v] * a01);
+                                    if (s10) atomic_add_f32(d_feats + o10 + ch + v, g[j][v] * a10);
+                                    if (s11) atomic_add_f32(d_feats + o11 + ch + v, g[j][v] * a11);
                                 }
                             }
                         }
                     }
                 }
-                if (d_depth != nullptr) {
+                if (need_G) {
                     // sum G over the lanes of the slot: lane `lis` adds lane `lis + off`
 #pragma unroll
                     for (int off = 32; off > 0; off >>= 1) {
                         float other = __shfl_down(G, off, kWave);
                         if (lis + off < k.lanes_per_slot) G += other;
                     }
-                    if (live && lis == 0) {
-                        const int kk = __float_as_int(dw.w);
-                        const int k0 = kk & 0xffff, k1 = kk >> 16;
-                        const float ga = G * dw.y, gb = G * dw.z;
-                        const size_t t00 = (size_t)__float_as_int(tf.x) * Dd, t01 = (size_t)__float_as_int(tf.y) * Dd;
-                        const size_t t10 = (size_t)__float_as_int(tf.z) * Dd, t11 = (size_t)__float_as_int(tf.w) * Dd;
-                        atomic_add_f32(d_depth + t00 + k0, ga * w.x);
-                        atomic_add_f32(d_depth + t00 + k1, gb * w.x);
-                        atomic_add_f32(d_depth + t01 + k0, ga * w.y);
-                        atomic_add_f32(d_depth + t01 + k1, gb * w.y);
-                        atomic_add_f32(d_depth + t10 + k0, ga * w.z);
-                        atomic_add_f32(d_depth + t10 + k1, gb * w.z);
-                        atomic_add_f32(d_depth + t11 + k0, ga * w.w);
-                        atomic_add_f32(d_depth + t11 + k1, gb * w.w);
+                }
+                if (live && lis == 0) {
+                    const int kk = __float_as_int(dw.w);
+                    const int k0 = kk & 0xffff, k1 = kk >> 16;
+                    const float ga = G * dw.y, gb = G * dw.z;
+                    const int t[4] = {__float_as_int(tf.x), __float_as_int(tf.y), __float_as_int(tf.z),
+                                      __float_as_int(tf.w)};
+                    const float wc[4] = {w.x, w.y, w.z, w.w};
+                    const int pos[4] = {__float_as_int(pf.x), __float_as_int(pf.y), __float_as_int(pf.z),
+                                        __float_as_int(pf.w)};
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const bool paired = FILL && pos[c] >= 0;
+                        if (paired && first_pass) {
+                            // G of a later channel pass cannot be folded into a pair already written:
+                            // passes after the first add their share of the depth gradient atomically.
+                            Pair pr;
+                            pr.cell = cell;
+                            pr.coef = wc[c] * dw.x * inv;
+                            pr.da = (need_G && parametric) ? ga * wc[c] : 0.0f;
+                            pr.db = (need_G && parametric) ? gb * wc[c] : 0.0f;
+                            *reinterpret_cast<float4 *>(pairs + pos[c]) =
+                                make_float4(__int_as_float(pr.cell), pr.coef, pr.da, pr.db);
+                        }
+                        if (need_G && !(paired && first_pass && parametric)) {
+                            atomic_add_f32(d_depth + (size_t)t[c] * Dd + k0, ga * wc[c]);
+                            atomic_add_f32(d_depth + (size_t)t[c] * Dd + k1, gb * wc[c]);
+                        }
                     }
                 }
             }
         }
         __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// Texel pass of the inverse-map backward: one block per texel.  Its 4 * (64 / lanes_per_row)
+// workers stride over the texel's pairs, each gathering grad_out rows with 128-bit loads;
+// partial rows meet in LDS and the block adds the sum to d_feats[texel, :] (and the depth
+// sums to d_depth[texel, 0:2]) with plain loads and stores -- the texel is owned by the block.
+template <int VEC>
+__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_kernel(
+    KParams k, const float *__restrict__ grad_out, const int *__restrict__ seg_end,
+    const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth, float *__restrict__ d_feats,
+    int lanes_per_row, int depth_from_pairs) {
+    extern __shared__ float4 smem[];
+    float *part = reinterpret_cast<float *>(smem);
+    const int t = blockIdx.x;
+    const int start = t == 0 ? 0 : seg_end[t - 1];
+    const int end = min(seg_end[t], pair_cap);
+    if (start >= end) return;      // uniform for the block
+    const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int wpw = kWave / lanes_per_row;            // workers per wavefront
+    const int nw = wpw * kWavesPerBlock;
+    const int wslot = lane / lanes_per_row;
+    const int lir = lane - wslot * lanes_per_row;
+    const bool worker_lane = wslot < wpw;
+    const int worker = wave * wpw + wslot;
+    const int span = lanes_per_row * VEC;
+    const int stride = span + 2;                      // partial row + the two depth sums
+    for (int c0 = 0; c0 < k.C; c0 += span) {
+        const int ch = c0 + lir * VEC;
+        const bool on = worker_lane && ch < k.C;
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+        float sa = 0.0f, sb = 0.0f;
+        if (on) {
+#pragma unroll 4
+            for (int e = start + worker; e < end; e += nw) {
+                const float4 pr = *reinterpret_cast<const float4 *>(pairs + e);
+                // a pair is written by the cell pass before this kernel starts; the range check
+                // only keeps a logic error from turning into a wild read
+                if ((unsigned)__float_as_int(pr.x) >= n_cells) continue;
+                const float *row = grad_out + (size_t)__float_as_int(pr.x) * k.C + ch;
+                if (VEC == 1) {
+                    acc[0] = __builtin_fmaf(pr.y, row[0], acc[0]);
+                } else {
+                    const float4 gq = *reinterpret_cast<const float4 *>(row);
+                    acc[0] = __builtin_fmaf(pr.y, gq.x, acc[0]);
+                    acc[1 % VEC] = __builtin_fmaf(pr.y, gq.y, acc[1 % VEC]);
+                    acc[2 % VEC] = __builtin_fmaf(pr.y, gq.z, acc[2 % VEC]);
+                    acc[3 % VEC] = __builtin_fmaf(pr.y, gq.w, acc[3 % VEC]);
+                }
+                sa += pr.z;
+                sb += pr.w;
+            }
+        }
+        __syncthreads();   // previous pass has been read
+        if (worker_lane) {
+            if (ch < k.C) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) part[worker * stride + lir * VEC + v] = acc[v];
+            }
+            if (lir == 0) {
+                part[worker * stride + span] = sa;
+                part[worker * stride + span + 1] = sb;
+            }
+        }
+        __syncthreads();
+        for (int c = threadIdx.x; c < span && c0 + c < k.C; c += blockDim.x) {
+            float sum = 0.0f;
+            for (int w = 0; w < nw; ++w) sum += part[w * stride + c];
+            if (d_feats != nullptr) d_feats[(size_t)t * k.C + c0 + c] += sum;
+        }
+        if (c0 == 0 && depth_from_pairs && threadIdx.x < 2) {
+            float sum = 0.0f;
+            for (int w = 0; w < nw; ++w) sum += part[w * stride + span + threadIdx.x];
+            d_depth[(size_t)t * 2 + threadIdx.x] += sum;
+        }
     }
 }
 
@@ -572,7 +781,7 @@ struct Plan {
     KParams k;
     int vec;        // elements per 16-byte load, or 1
     int cpl;        // channel vectors per lane per pass
-    size_t lds_fwd, lds_bwd;
+    size_t lds_fwd, lds_bwd, lds_fill;
 };
 
 int elem_size(int dtype) { return dtype == FBEV_F32 ? 4 : 2; }
@@ -632,8 +841,8 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan) {
     plan->cpl = cpl;
     k.lanes_per_slot = lps;
     int slots = kWave / lps;
-    // lists of both kernels must fit the per-wave LDS budget (3 float4 per entry in backward)
-    const int entry_bytes = 48;
+    // lists of all kernels must fit the per-wave LDS budget (up to 4 float4 per entry in backward)
+    const int entry_bytes = 64;
     while (slots > 1 && (long long)slots * k.NZ * entry_bytes > kMaxSlotLdsBytes) --slots;
     if (slots > 16) slots = 16;
     k.slots = slots;
@@ -648,7 +857,8 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan) {
     const size_t p_f4 = (size_t)(k.N * 12 + 3) / 4;
     plan->lds_fwd = (p_f4 + (size_t)kWavesPerBlock * (4 + (size_t)k.slots * k.list_cap * 2)) * 16;
     plan->lds_bwd = (p_f4 + (size_t)kWavesPerBlock * (4 + (size_t)k.slots * k.list_cap * 3)) * 16;
-    if (plan->lds_bwd > (size_t)kMaxBlockLdsBytes) return FBEV_ERR_TOO_LARGE;
+    plan->lds_fill = (p_f4 + (size_t)kWavesPerBlock * (4 + (size_t)k.slots * k.list_cap * 4)) * 16;
+    if (plan->lds_fill > (size_t)kMaxBlockLdsBytes) return FBEV_ERR_TOO_LARGE;
     return FBEV_OK;
 }
 
@@ -666,18 +876,65 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
-template <typename T, int VEC>
-int launch_backward(const Plan &pl, const float *go, const void *depth, const void *feats, const float *proj,
-                    float *dd, float *df, hipStream_t st) {
+template <typename T, int VEC, bool FILL>
+int launch_cells(const Plan &pl, const float *go, const void *depth, const void *feats, const float *proj,
+                 float *dd, float *df, int *cursor, Pair *pairs, int cap, hipStream_t st) {
     dim3 grid(pl.k.n_blocks), block(kWave * kWavesPerBlock);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
+    const size_t lds = FILL ? pl.lds_fill : pl.lds_bwd;
     switch (pl.cpl) {
-        case 1: hipLaunchKernelGGL((fbev_backward_kernel<T, VEC, 1>), grid, block, pl.lds_bwd, st, pl.k, go, d, f, proj, dd, df); break;
-        case 2: hipLaunchKernelGGL((fbev_backward_kernel<T, VEC, 2>), grid, block, pl.lds_bwd, st, pl.k, go, d, f, proj, dd, df); break;
-        default: hipLaunchKernelGGL((fbev_backward_kernel<T, VEC, 4>), grid, block, pl.lds_bwd, st, pl.k, go, d, f, proj, dd, df); break;
+        case 1: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, cursor, pairs, cap); break;
+        case 2: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, cursor, pairs, cap); break;
+        default: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, cursor, pairs, cap); break;
     }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+template <bool FILL>
+int dispatch_cells(const fbev_problem *p, const Plan &pl, const float *go, const void *depth, const void *feats,
+                   const float *proj, float *dd, float *df, int *cursor, Pair *pairs, int cap, hipStream_t st) {
+    switch (p->in_dtype) {
+        case FBEV_F32:
+            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st)
+                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st);
+        case FBEV_F16:
+            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st)
+                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st);
+        default:
+            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st)
+                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st);
+    }
+}
+
+template <typename T>
+int launch_count(const Plan &pl, const void *depth, const float *proj, int *counts, long long total, hipStream_t st) {
+    hipLaunchKernelGGL((fbev_count_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, pl.k,
+                       static_cast<const T *>(depth), proj, counts, total);
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+long long texel_count(const fbev_problem *p) {
+    return (long long)p->batch * p->num_cams * p->feat_h * p->feat_w;
+}
+
+long long sample_count(const fbev_problem *p) {
+    return (long long)p->batch * p->grid_y * p->grid_x * p->num_cams * p->grid_z;
+}
+
+// Workspace layout: [texels + 1 int32 segment cursors, padded to 256 bytes][pairs]
+size_t ws_index_bytes(const fbev_problem *p) {
+    return (((size_t)texel_count(p) + 1) * sizeof(int) + 255) / 256 * 256;
+}
+
+int check_backward_args(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                        const float *proj, const float *d_depth, const float *d_feats) {
+    if (!grad_out || !depth || !feats || !proj) return FBEV_ERR_NULL;
+    const int es = elem_size(p->in_dtype);
+    if ((uintptr_t)depth % es || (uintptr_t)feats % es || (uintptr_t)proj % 4 || (uintptr_t)grad_out % 4 ||
+        (uintptr_t)d_depth % 4 || (uintptr_t)d_feats % 4)
+        return FBEV_ERR_ALIGNMENT;
+    return FBEV_OK;
 }
 
 }  // namespace
@@ -714,27 +971,79 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
                   const float *proj, float *d_depth, float *d_feats, void *stream) {
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
-    if (!grad_out || !depth || !feats || !proj) return FBEV_ERR_NULL;
+    rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
+    if (rc != FBEV_OK) return rc;
     if (!d_depth && !d_feats) return FBEV_OK;
-    const int es = elem_size(p->in_dtype);
-    if ((uintptr_t)depth % es || (uintptr_t)feats % es || (uintptr_t)proj % 4 || (uintptr_t)grad_out % 4 ||
-        (uintptr_t)d_depth % 4 || (uintptr_t)d_feats % 4)
-        return FBEV_ERR_ALIGNMENT;
+    Plan pl;
+    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl);
+    if (rc != FBEV_OK) return rc;
+    return dispatch_cells<false>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, nullptr, nullptr, 0,
+                                 static_cast<hipStream_t>(stream));
+}
+
+uint64_t fbev_backward_max_pairs(const fbev_problem *p) {
+    if (validate(p, true) != FBEV_OK) return 0;
+    return 4ull * (uint64_t)sample_count(p);
+}
+
+size_t fbev_backward_workspace_bytes(const fbev_problem *p, uint64_t pair_capacity) {
+    if (validate(p, true) != FBEV_OK) return 0;
+    return ws_index_bytes(p) + (size_t)pair_capacity * sizeof(Pair);
+}
+
+int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                         const float *proj, float *d_depth, float *d_feats, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    int rc = validate(p, true);
+    if (rc != FBEV_OK) return rc;
+    rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
+    if (rc != FBEV_OK) return rc;
+    if (!d_depth && !d_feats) return FBEV_OK;
+    if (!workspace) return FBEV_ERR_NULL;
+    if ((uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
+    const size_t index_bytes = ws_index_bytes(p);
+    if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
+    // pair positions are 32-bit: every sample corner must be countable
+    if (4 * sample_count(p) >= (1ll << 31) || texel_count(p) + 1 >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    size_t cap64 = (workspace_bytes - index_bytes) / sizeof(Pair);
+    const int cap = cap64 > 0x7fffffffull ? 0x7fffffff : (int)cap64;
     Plan pl;
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl);
     if (rc != FBEV_OK) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    int *cursor = static_cast<int *>(workspace);
+    Pair *pairs = reinterpret_cast<Pair *>(static_cast<char *>(workspace) + index_bytes);
+    const long long texels = texel_count(p), samples = sample_count(p);
+
+    hipLaunchKernelGGL(fbev_fill_zero_kernel, dim3((unsigned)((texels + 1 + 255) / 256)), dim3(256), 0, st, cursor,
+                       texels + 1);
+    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
     switch (p->in_dtype) {
-        case FBEV_F32:
-            return pl.vec == 4 ? launch_backward<float, 4>(pl, grad_out, depth, feats, proj, d_depth, d_feats, st)
-                               : launch_backward<float, 1>(pl, grad_out, depth, feats, proj, d_depth, d_feats, st);
-        case FBEV_F16:
-            return pl.vec == 8 ? launch_backward<__half, 8>(pl, grad_out, depth, feats, proj, d_depth, d_feats, st)
-                               : launch_backward<__half, 1>(pl, grad_out, depth, feats, proj, d_depth, d_feats, st);
-        default:
-            return pl.vec == 8 ? launch_backward<bf16_raw, 8>(pl, grad_out, depth, feats, proj, d_depth, d_feats, st)
-                               : launch_backward<bf16_raw, 1>(pl, grad_out, depth, feats, proj, d_depth, d_feats, st);
+        case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, samples, st); break;
+        case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, samples, st); break;
+        default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, samples, st); break;
     }
+    if (rc != FBEV_OK) return rc;
+    hipLaunchKernelGGL(fbev_scan_kernel, dim3(1), dim3(1024), 0, st, cursor, (int)texels);
+    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+    rc = dispatch_cells<true>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, cursor, pairs, cap, st);
+    if (rc != FBEV_OK) return rc;
+
+    // texel pass: rows of grad_out are fp32, so 128-bit gathers need C % 4 == 0 and aligned rows
+    const bool vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
+    const int vec = vec4 ? 4 : 1;
+    const int cq = (p->channels + vec - 1) / vec;
+    const int lpr = cq < kWave ? cq : kWave;
+    const int nw = (kWave / lpr) * kWavesPerBlock;
+    const size_t lds = (size_t)nw * (lpr * vec + 2) * sizeof(float);
+    const int from_pairs = (d_depth != nullptr && p->depth_distribution != FBEV_CATEGORICAL) ? 1 : 0;
+    if (vec4)
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels), dim3(kWave * kWavesPerBlock), lds,
+                           st, pl.k, grad_out, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
+    else
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels), dim3(kWave * kWavesPerBlock), lds,
+                           st, pl.k, grad_out, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
 int fbev_sample_geometry(const fbev_problem *p, const float *proj, uint8_t *mask, int32_t *idx, float *frac,

@@ -172,7 +172,8 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                             const at::Tensor &image_size, const at::Tensor &roi_range, const at::Tensor &grid_size,
                             std::optional<at::Tensor> depth_params_grad, std::optional<at::Tensor> image_feats_grad,
                             int64_t total_threads, int depth_distribution, float epsilon, float depth_weight_threshold,
-                            float depth_min, float depth_step, int reduction) {
+                            float depth_min, float depth_step, int reduction, int backward_mode,
+                            int64_t pair_capacity) {
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
     auto roi = host_floats(roi_range, 6, "roi_range");
@@ -204,9 +205,25 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
     }
     DeviceScope scope(depth_params.get_device());
     hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
-    raise_on(fbev_backward(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
-                           projection_matrices.data_ptr<float>(), dd, df, st),
-             "fbev_backward");
+    TORCH_CHECK(backward_mode >= 0 && backward_mode <= 2,
+                "flashbevpool_ext: backward_mode must be 0 (auto), 1 (atomic scatter) or 2 (inverse-map gather)");
+    if (backward_mode == 1) {
+        raise_on(fbev_backward(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                               projection_matrices.data_ptr<float>(), dd, df, st),
+                 "fbev_backward");
+        return;
+    }
+    // Inverse-map gather.  The pair array comes from PyTorch's caching allocator (no device
+    // allocation in steady state).  Half of the worst case holds every rig whose cameras see
+    // less than half of all (cell, height) samples; what does not fit is applied with atomics.
+    const uint64_t max_pairs = fbev_backward_max_pairs(&p);
+    uint64_t cap = pair_capacity >= 0 ? (uint64_t)pair_capacity : (max_pairs + 1) / 2;
+    if (cap > max_pairs) cap = max_pairs;
+    const size_t bytes = fbev_backward_workspace_bytes(&p, cap);
+    at::Tensor ws = at::empty({(int64_t)bytes}, at::TensorOptions().device(depth_params.device()).dtype(at::kByte));
+    raise_on(fbev_backward_gather(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                                  projection_matrices.data_ptr<float>(), dd, df, ws.data_ptr(), bytes, st),
+             "fbev_backward_gather");
 }
 
 // Parity hook: per-sample validity mask and bilinear corner indices, [B,gy,gx,N,gz(,4|2)].
@@ -261,7 +278,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("feature_size"), py::arg("image_size"), py::arg("roi_range"), py::arg("grid_size"),
           py::arg("depth_params_grad"), py::arg("image_feats_grad"), py::arg("total_threads"),
           py::arg("depth_distribution"), py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f,
-          py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0);
+          py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0,
+          py::arg("backward_mode") = 0, py::arg("pair_capacity") = -1);
     m.def("sample_geometry", &sample_geometry, "per-sample validity mask and corner indices (parity hook)",
           py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
           py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);

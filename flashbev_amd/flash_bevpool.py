@@ -23,6 +23,7 @@ results in the reference either.
 """
 from __future__ import annotations
 
+import os
 import weakref
 from typing import Sequence
 
@@ -32,6 +33,16 @@ import torch
 from ._native import load_ext
 
 _SUPPORTED = (torch.float32, torch.float16, torch.bfloat16)
+# how the backward pass forms the feature gradient: "gather" (inverse map, no float atomics,
+# the default) or "scatter" (hardware fp32 atomics, no workspace)
+_BACKWARD_MODES = {"auto": 0, "scatter": 1, "gather": 2}
+
+
+def _backward_mode() -> int:
+    name = os.environ.get("FLASHBEV_BACKWARD", "auto").lower()
+    if name not in _BACKWARD_MODES:
+        raise ValueError(f"FLASHBEV_BACKWARD must be one of {sorted(_BACKWARD_MODES)}, got {name!r}")
+    return _BACKWARD_MODES[name]
 _host_cache: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()
 
 
@@ -147,7 +158,7 @@ class FlashBEVPool(torch.autograd.Function):
                 out_grad.contiguous().float(), depth_params, image_feats, projection_matrices,
                 fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
                 ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
-                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction)
+                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, _backward_mode(), -1)
         return (depth_params_grad, image_feats_grad) + (None,) * 14
 
 

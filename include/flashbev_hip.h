@@ -95,6 +95,32 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
                   const float *proj, float *d_depth, float *d_feats, void *stream);
 
 /*
+ * Backward through an inverse map (texel -> contributing samples): the same gradients as
+ * fbev_backward, formed without floating-point atomics on the feature gradient.  The call
+ * counts the contributing sample corners per texel, prefix-sums the counts, writes one
+ * 16-byte (cell, coefficient) pair per corner into the texel's segment of the workspace and
+ * then gathers per texel.  It ACCUMULATES into the zero-filled d_depth / d_feats like
+ * fbev_backward.  `workspace` is caller-owned device memory, 16-byte aligned, of at least
+ * fbev_backward_workspace_bytes(p, 0) bytes; pairs that do not fit its capacity are applied
+ * with atomics instead, so any capacity gives correct results and
+ * fbev_backward_workspace_bytes(p, fbev_backward_max_pairs(p)) never overflows.  The
+ * workspace carries no state between calls.
+ * It is the deterministic-gather alternative to the atomic scatter of
+ * flash_bevpool_grad_kernel (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:570-681); the sorted
+ * (cell -> sample) intervals of flashbev/flashbevpool/sampling_vt.py:296-311 are the same idea
+ * applied to the forward pass.
+ */
+int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                         const float *proj, float *d_depth, float *d_feats, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
+/* Upper bound of the pairs one backward call can produce: 4 corners per (cell, camera, height) sample. */
+uint64_t fbev_backward_max_pairs(const fbev_problem *p);
+
+/* Bytes of a workspace holding the per-texel index plus `pair_capacity` pairs. */
+size_t fbev_backward_workspace_bytes(const fbev_problem *p, uint64_t pair_capacity);
+
+/*
  * Inspection hook for parity tests: per (b, y, x, camera, height-bin) sample, in that
  * order, the projection validity and the bilinear corner indices the kernels use.
  *   mask  uint8  [B,gy,gx,N,gz]      1 = depth > 0 and inside the feature map

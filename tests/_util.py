@@ -73,16 +73,28 @@ def capi_forward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN
     return out
 
 
-def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, want=(True, True)):
+def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, want=(True, True),
+                  mode="scatter", pair_capacity=None):
+    """Backward through the C ABI.  mode "scatter" = fbev_backward, "gather" = fbev_backward_gather
+    with a workspace for `pair_capacity` pairs (default: the worst case)."""
     p = problem_for(x, w, dist, thr, eps, reduction)
     dev = x["image_feats"].device
     dd = torch.zeros(x["depth_params"].shape, dtype=torch.float32, device=dev) if want[0] else None
     df = torch.zeros(x["image_feats"].shape, dtype=torch.float32, device=dev) if want[1] else None
     st = torch.cuda.current_stream().cuda_stream
-    capi.check(capi.backward(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
-                             x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(),
-                             dd.data_ptr() if dd is not None else None,
-                             df.data_ptr() if df is not None else None, st), "fbev_backward")
+    ddp = dd.data_ptr() if dd is not None else None
+    dfp = df.data_ptr() if df is not None else None
+    if mode == "scatter":
+        capi.check(capi.backward(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
+                                 x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(), ddp, dfp, st),
+                   "fbev_backward")
+    else:
+        cap = capi.backward_max_pairs(p) if pair_capacity is None else pair_capacity
+        nbytes = capi.backward_workspace_bytes(p, cap)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        capi.check(capi.backward_gather(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
+                                        x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(), ddp, dfp,
+                                        ws.data_ptr(), nbytes, st), "fbev_backward_gather")
     torch.cuda.synchronize()
     return dd, df
 

@@ -56,13 +56,35 @@ def test_forward_matches_c_oracle(name, dist, thr):
 
 @pytest.mark.parametrize("name", ["cfg1_tiny", "cfg2_surround"])
 @pytest.mark.parametrize("dist", [0, 1, 2])
-def test_backward_matches_c_oracle(name, dist):
+@pytest.mark.parametrize("mode", ["scatter", "gather"])
+def test_backward_matches_c_oracle(name, dist, mode):
     w, x = _inputs(name, dist)
-    dd, df = U.capi_backward(x, w, dist)
+    dd, df = U.capi_backward(x, w, dist, mode=mode)
     want_dd, want_df = U.oracle_backward(x, w, dist)
     for got, want, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
         bad, maxabs, ratio = U.violations(got.cpu().numpy(), want)
         assert bad == 0, f"{what}: {bad} elements outside tolerance, max |diff| {maxabs:.3e}, ratio {ratio:.2f}"
+
+
+@pytest.mark.parametrize("capacity", [0, 1000, 100000])
+def test_backward_gather_with_short_workspace(capacity):
+    """Pairs that do not fit the workspace are applied with atomics: any capacity is correct."""
+    w, x = _inputs("cfg2_surround", 1)
+    dd, df = U.capi_backward(x, w, 1, mode="gather", pair_capacity=capacity)
+    want_dd, want_df = U.oracle_backward(x, w, 1)
+    assert U.violations(df.cpu().numpy(), want_df)[0] == 0
+    assert U.violations(dd.cpu().numpy(), want_dd)[0] == 0
+
+
+def test_backward_single_gradient():
+    """Either gradient pointer may be NULL."""
+    w, x = _inputs("cfg2_surround", 0)
+    want_dd, want_df = U.oracle_backward(x, w, 0)
+    for mode in ("scatter", "gather"):
+        dd, df = U.capi_backward(x, w, 0, mode=mode, want=(True, False))
+        assert df is None and U.violations(dd.cpu().numpy(), want_dd)[0] == 0
+        dd, df = U.capi_backward(x, w, 0, mode=mode, want=(False, True))
+        assert dd is None and U.violations(df.cpu().numpy(), want_df)[0] == 0
 
 
 @pytest.mark.parametrize("dist", [0, 1])
@@ -78,7 +100,7 @@ def test_forward_backward_vs_dense_torch(dist):
                                                    cpu["projection_matrices"].double(),
                                                    cpu["grad_out"].double(), **kw)
     out = U.capi_forward(x, w, dist).cpu()
-    dd, df = U.capi_backward(x, w, dist)
+    dd, df = U.capi_backward(x, w, dist, mode="gather")
     for got, r32, r64, what in ((out, o32, o64, "out"), (df.cpu(), df32, df64, "d_feats"),
                                 (dd.cpu(), dd32, dd64, "d_depth")):
         bad, maxabs, ratio = U.violations(got.numpy(), r32.numpy())
@@ -91,8 +113,10 @@ def test_forward_backward_vs_dense_torch(dist):
         # relative condition number z^2 up to ~27): a few elements leave the band in both
         assert bad <= 2e-2 * got.numel()
         assert ours_ratio <= 4.0 * max(floor_ratio, 1.0)
-        m = U.reference_metrics(got.numpy(), r32.numpy())
-        assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["cosine"] > 0.9999, m
+        if what == "out":
+            # the reference's own (forward-only) acceptance statistics, tools/profile_differences.py:70-106
+            m = U.reference_metrics(got.numpy(), r32.numpy())
+            assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["mean_rel"] < 1e-3 and m["cosine"] > 0.9999, m
 
 
 def test_autograd_operator_matches_capi():
