@@ -9,9 +9,11 @@ extension module.  The default workload is the 6-camera 128x128x8 fp32 configura
 (``cfg2_surround``) with the reference benchmark's depth model (per-pixel Laplace
 parameters, tools/config/config.yaml:29).  The single JSON line printed on stdout carries
   value / ms_per_step   forward+backward latency per step (ms)
-  roofline              dominant kernel: compulsory bytes of that kernel / its mean duration
-                        (HIP events recorded around every launch in the timed region),
-                        against the 8 TB/s HBM3E peak
+  roofline              the dominant pass (the backward, five kernel launches): its compulsory
+                        bytes / the summed mean durations of its kernels, measured with HIP
+                        events the library records around every one of its launches over a
+                        second run of the same K steps, against the 8 TB/s HBM3E peak;
+                        "kernels" lists every kernel's mean duration and launch count
   cpu_baseline          the dense PyTorch restatement of the reference's pooling path
                         (oracle/dense_torch.py), forward+backward via autograd on the host
                         cores, same workload -- a reported baseline, not a target.
@@ -32,6 +34,7 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from flashbev_amd import capi  # noqa: E402
 from flashbev_amd._native import load_ext  # noqa: E402
 from flashbev_amd.flash_bevpool import voxel_geometry  # noqa: E402
 from flashbev_amd.workloads import WORKLOADS, algorithmic_bytes, make_inputs  # noqa: E402
@@ -103,6 +106,21 @@ def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
     fwd = [ev[i][0].elapsed_time(ev[i][1]) for i in range(steps)]
     bwd = [ev[i][2].elapsed_time(ev[i][3]) for i in range(steps)] if with_backward else []
     return (t1 - t0) * 1e3 / steps, fwd, bwd
+
+
+def profile_steps(r: Runner, steps: int):
+    """The same steps again with the library's per-kernel event timing switched on."""
+    capi.profile_enable(True)
+    try:
+        for _ in range(steps):
+            r.forward()
+            r.zero_grads()
+            r.backward()
+        torch.cuda.synchronize()
+        got = capi.profile_collect()
+    finally:
+        capi.profile_enable(False)
+    return {name: {"mean_us": ms / calls * 1e3, "calls_per_step": calls / steps} for name, (ms, calls) in got.items()}
 
 
 def cpu_baseline(w, depth_name: str, budget_s: float = 20.0, max_runs: int = 5):
@@ -182,6 +200,10 @@ def main():
     ap.add_argument("--depth", default="laplace", choices=sorted(DIST_OF))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--table", action="store_true")
+    ap.add_argument("--backward-mode", type=int, default=0, choices=(0, 1, 2),
+                    help="0/2 inverse-map gather (default), 1 atomic scatter")
+    ap.add_argument("--pmc-copy-mib", type=int, default=0,
+                    help="only run a device-to-device copy of this many MiB (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; batch elements are independent, so more GPUs "
@@ -192,13 +214,29 @@ def main():
         sys.exit(3)
     torch.cuda.set_device(0)
     w = WORKLOADS[args.workload]
-    r = Runner(w, args.depth)
+    if args.pmc_copy_mib:
+        # calibration for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: one device-to-device copy of known size
+        n = args.pmc_copy_mib << 20
+        src = torch.ones(n, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n}))
+        return
+    r = Runner(w, args.depth, backward_mode=args.backward_mode)
     ms, fwd, bwd = time_steps(r, args.steps, args.warmup, True)
+    kernels = profile_steps(r, args.steps)
     fwd_ms, bwd_ms = statistics.mean(fwd), statistics.mean(bwd)
     fb, bb = algorithmic_bytes(w, r.model, False), algorithmic_bytes(w, r.model, True)
-    dominant = "backward" if bwd_ms >= fwd_ms else "forward"
-    k_ms, k_bytes = (bwd_ms, bb) if dominant == "backward" else (fwd_ms, fb)
+    fwd_names = [k for k in kernels if "forward" in k]
+    bwd_names = [k for k in kernels if k not in fwd_names]
+    fwd_k_ms = sum(kernels[k]["mean_us"] * kernels[k]["calls_per_step"] for k in fwd_names) / 1e3
+    bwd_k_ms = sum(kernels[k]["mean_us"] * kernels[k]["calls_per_step"] for k in bwd_names) / 1e3
+    dominant = "backward" if bwd_k_ms >= fwd_k_ms else "forward"
+    k_ms, k_bytes, k_names = (bwd_k_ms, bb, bwd_names) if dominant == "backward" else (fwd_k_ms, fb, fwd_names)
     achieved = k_bytes / k_ms / 1e6  # GB/s
+    top = max(kernels, key=lambda k: kernels[k]["mean_us"] * kernels[k]["calls_per_step"])
     line = {
         "metric": "BEV-pool fwd+bwd latency (ms) & effective HBM GB/s, 6 cams 128x128xZ=8, 1 GPU",
         "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -207,13 +245,18 @@ def main():
         "data": "synthetic",
         "config": {"workload": w.name, "depth_model": args.depth, "batch": w.batch, "cams": w.num_cams,
                    "channels": w.channels, "feat_hw": list(w.feat_hw), "grid": list(w.grid_size),
-                   "step": "forward kernel + zero-fill of both gradient buffers + backward kernel"},
-        "fwd_kernel_ms": stats(fwd), "bwd_kernel_ms": stats(bwd),
+                   "backward": {0: "inverse-map gather", 1: "atomic scatter", 2: "inverse-map gather"}[args.backward_mode],
+                   "step": "forward kernel + zero-fill of both gradient buffers + backward kernels"},
+        "fwd_call_ms": stats(fwd), "bwd_call_ms": stats(bwd),
         "effective_GBps_fwd_bwd": (fb + bb) / ms / 1e6,
         "frac_hbm_fwd_bwd": (fb + bb) / ms / 1e6 / HBM_PEAK_GBS,
-        "roofline": {"bound": "hbm", "kernel": f"fbev_{dominant}_kernel", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes": k_bytes, "kernel_ms": k_ms},
+        "kernels": kernels,
+        "roofline": {"bound": "hbm", "kernel": f"{dominant} pass = " + " + ".join(k_names),
+                     "dominant_kernel": top, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": k_bytes,
+                     "kernel_ms": k_ms,
+                     "forward": {"algorithmic_bytes": fb, "kernel_ms": fwd_k_ms,
+                                 "frac": fb / fwd_k_ms / 1e6 / HBM_PEAK_GBS if fwd_k_ms else None}},
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, args.depth)

@@ -17,7 +17,8 @@ FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
 EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_max_pairs",
            "fbev_backward_workspace_bytes", "fbev_sample_geometry", "fbev_algorithmic_bytes",
-           "fbev_status_string", "fbev_abi_version", "fbev_problem_size")
+           "fbev_profile_enable", "fbev_profile_kernel_count", "fbev_profile_kernel_name",
+           "fbev_profile_collect", "fbev_status_string", "fbev_abi_version", "fbev_problem_size")
 
 
 class FbevProblem(ctypes.Structure):
@@ -56,6 +57,13 @@ def load() -> ctypes.CDLL:
         lib.fbev_sample_geometry.restype = ctypes.c_int
         lib.fbev_algorithmic_bytes.argtypes = [pp, ctypes.c_int]
         lib.fbev_algorithmic_bytes.restype = ctypes.c_uint64
+        lib.fbev_profile_enable.argtypes = [ctypes.c_int]
+        lib.fbev_profile_enable.restype = ctypes.c_int
+        lib.fbev_profile_kernel_count.restype = ctypes.c_int
+        lib.fbev_profile_kernel_name.argtypes = [ctypes.c_int]
+        lib.fbev_profile_kernel_name.restype = ctypes.c_char_p
+        lib.fbev_profile_collect.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]
+        lib.fbev_profile_collect.restype = ctypes.c_int
         lib.fbev_status_string.argtypes = [ctypes.c_int]
         lib.fbev_status_string.restype = ctypes.c_char_p
         lib.fbev_abi_version.restype = ctypes.c_int
@@ -139,3 +147,17 @@ def sample_geometry(p: FbevProblem, proj_ptr: int, mask_ptr: Optional[int], idx_
 
 def algorithmic_bytes(p: FbevProblem, backward_pass: bool) -> int:
     return int(load().fbev_algorithmic_bytes(ctypes.byref(p), int(bool(backward_pass))))
+
+
+def profile_enable(on: bool) -> None:
+    check(load().fbev_profile_enable(int(bool(on))), "fbev_profile_enable")
+
+
+def profile_collect() -> dict:
+    """{kernel name: (total_ms, calls)} of the launches recorded since profiling was enabled."""
+    lib = load()
+    n = lib.fbev_profile_kernel_count()
+    ms = (ctypes.c_double * n)()
+    calls = (ctypes.c_int64 * n)()
+    check(lib.fbev_profile_collect(ms, calls), "fbev_profile_collect")
+    return {lib.fbev_profile_kernel_name(i).decode(): (ms[i], int(calls[i])) for i in range(n) if calls[i]}

@@ -25,15 +25,61 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <mutex>
+#include <vector>
+
 #include "flashbev_hip.h"
 
 namespace {
+
+// ---------------------------------------------------------------- per-kernel timing (opt-in)
+// While enabled, every kernel launch of this library is bracketed by a pair of HIP events
+// on the launch stream; fbev_profile_collect() waits for them and returns total time and
+// call count per kernel.  Disabled (the default) it costs one relaxed atomic load per launch.
+namespace prof {
+enum Kid { kForward, kBackwardScatter, kZero, kCount, kScanChunks, kScanSums, kBackwardCells, kBackwardTexel,
+           kGeometry, kNum };
+const char *const kNames[kNum] = {"fbev_forward_kernel", "fbev_backward_cells_kernel<scatter>",
+                                  "fbev_fill_zero_kernel", "fbev_count_kernel", "fbev_scan_chunks_kernel",
+                                  "fbev_scan_sums_kernel", "fbev_backward_cells_kernel<fill>",
+                                  "fbev_backward_texel_kernel", "fbev_geometry_kernel"};
+struct Rec { hipEvent_t a, b; int kid; };
+std::atomic<bool> enabled{false};
+std::mutex mu;
+std::vector<Rec> recs;
+
+struct Scope {
+    hipStream_t st;
+    Rec r;
+    bool live;
+    Scope(int kid, hipStream_t s) : st(s), live(enabled.load(std::memory_order_relaxed)) {
+        if (!live) return;
+        r.kid = kid;
+        if (hipEventCreate(&r.a) != hipSuccess || hipEventCreate(&r.b) != hipSuccess) { live = false; return; }
+        (void)hipEventRecord(r.a, st);
+    }
+    ~Scope() {
+        if (!live) return;
+        (void)hipEventRecord(r.b, st);
+        std::lock_guard<std::mutex> g(mu);
+        recs.push_back(r);
+    }
+};
+}  // namespace prof
 
 constexpr int kWave = 64;
 constexpr int kWavesPerBlock = 4;
 constexpr int kTile = 8;            // BEV cells are walked in 8x8 tiles for gather locality
 constexpr int kMaxSlotLdsBytes = 12 * 1024;  // per-wave budget for the compacted lists
 constexpr int kMaxBlockLdsBytes = 64 * 1024; // dynamic LDS a block may ask for without opting in
+constexpr int kXcdCount = 8;                 // accelerator complex dies, each with its own L2
+// The inverse map counts sample corners per texel with integer atomics.  Atomics on one
+// address execute one after the other, and the texels on the horizon collect thousands of
+// samples, so every texel owns kReplicas counters and a sample picks one from its cell.
+constexpr int kReplicaBits = 5;
+constexpr int kReplicas = 1 << kReplicaBits;
+constexpr int kScanChunkBits = 12;           // counters are prefix-summed in chunks of 4096
 
 struct KParams {
     int B, N, H, W, C;
@@ -216,12 +262,14 @@ __device__ __forceinline__ bool cell_of(const KParams &k, int q, int &ix, int &i
 // Blocks are dealt round-robin to the 8 XCDs; renumber them so that each XCD walks one
 // contiguous range of (batch, tile) space and its L2 keeps one batch element's maps.
 __device__ __forceinline__ int xcd_swizzle(int bid, int n_blocks) {
-    constexpr int kXcd = 8;
+    constexpr int kXcd = kXcdCount;
     int per = n_blocks / kXcd;
     int main = per * kXcd;
     if (bid >= main) return bid;
     return (bid % kXcd) * per + bid / kXcd;
 }
+
+__device__ __forceinline__ int replica_of(int ix, int iy) { return (ix + 5 * iy) & (kReplicas - 1); }
 
 __device__ __forceinline__ unsigned long long lanemask_lt(int lane) {
     return lane == 0 ? 0ull : (~0ull >> (64 - lane));
@@ -239,6 +287,7 @@ enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2 };
 template <int ENTRY_F4, typename T, int MODE>
 __device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const T *__restrict__ depth,
                                         int b, int q0, int lane, float4 *lst, volatile int *cnt,
+                                        const int *__restrict__ chunk_prefix = nullptr,
                                         int *__restrict__ cursor = nullptr, int pair_cap = 0) {
     constexpr bool BACKWARD = MODE != kModeForward;
     const int total = k.slots * k.NZ;
@@ -295,10 +344,17 @@ __device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const
             if (MODE == kModeFill) {
                 // claim one slot per corner in the texel's segment of the pair array; the four
                 // requests of all lanes are in flight together, so the round trip is paid once
-                int p0 = atomicAdd(cursor + tx.x, 1);
-                int p1 = atomicAdd(cursor + tx.y, 1);
-                int p2 = atomicAdd(cursor + tx.z, 1);
-                int p3 = atomicAdd(cursor + tx.w, 1);
+                const int rep = replica_of(ix, iy);
+                const int i0 = tx.x * kReplicas + rep, i1 = tx.y * kReplicas + rep;
+                const int i2 = tx.z * kReplicas + rep, i3 = tx.w * kReplicas + rep;
+                int p0 = atomicAdd(cursor + i0, 1);
+                int p1 = atomicAdd(cursor + i1, 1);
+                int p2 = atomicAdd(cursor + i2, 1);
+                int p3 = atomicAdd(cursor + i3, 1);
+                p0 += chunk_prefix[i0 >> kScanChunkBits];
+                p1 += chunk_prefix[i1 >> kScanChunkBits];
+                p2 += chunk_prefix[i2 >> kScanChunkBits];
+                p3 += chunk_prefix[i3 >> kScanChunkBits];
                 p0 = p0 < pair_cap ? p0 : -1;
                 p1 = p1 < pair_cap ? p1 : -1;
                 p2 = p2 < pair_cap ? p2 : -1;
@@ -468,14 +524,44 @@ __global__ __launch_bounds__(256) void fbev_count_kernel(KParams k, const T *__r
     int t11 = (rowbase + g.v1) * k.W + g.u1;
     DepthEval e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
     if (!e.keep) return;
-    atomicAdd(counts + t00, 1);
-    atomicAdd(counts + t01, 1);
-    atomicAdd(counts + t10, 1);
-    atomicAdd(counts + t11, 1);
+    const int rep = replica_of(ix, iy);
+    atomicAdd(counts + t00 * kReplicas + rep, 1);
+    atomicAdd(counts + t01 * kReplicas + rep, 1);
+    atomicAdd(counts + t10 * kReplicas + rep, 1);
+    atomicAdd(counts + t11 * kReplicas + rep, 1);
 }
 
-// In-place exclusive prefix sum of v[0..n) by one block; v[n] receives the total.
-__global__ __launch_bounds__(1024) void fbev_scan_kernel(int *v, int n) {
+// Prefix sum of the counters in two launches.  (1) Every block turns its chunk of 4096
+// counters into exclusive prefix sums within the chunk and records the chunk total.
+// (2) One block turns the chunk totals into exclusive prefix sums.  A counter's global
+// position is chunk_prefix[i >> 12] + v[i]; nobody needs it materialised.
+__global__ __launch_bounds__(1024) void fbev_scan_chunks_kernel(int *__restrict__ v, long long n,
+                                                                int *__restrict__ chunk_sums) {
+    __shared__ int part[1024];
+    const int tid = threadIdx.x;
+    const long long base = ((long long)blockIdx.x << kScanChunkBits) + tid * 4;
+    int c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c[j] = base + j < n ? v[base + j] : 0;
+    const int sum = c[0] + c[1] + c[2] + c[3];
+    part[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        int add = tid >= off ? part[tid - off] : 0;
+        __syncthreads();
+        part[tid] += add;
+        __syncthreads();
+    }
+    int run = part[tid] - sum;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (base + j < n) v[base + j] = run;
+        run += c[j];
+    }
+    if (tid == 1023) chunk_sums[blockIdx.x] = part[1023];
+}
+
+__global__ __launch_bounds__(1024) void fbev_scan_sums_kernel(int *v, int n) {
     __shared__ int part[1024];
     const int tid = threadIdx.x;
     const int chunk = (n + 1023) / 1024;
@@ -496,17 +582,16 @@ __global__ __launch_bounds__(1024) void fbev_scan_kernel(int *v, int n) {
         v[i] = run;
         run += c;
     }
-    if (tid == 1023) v[n] = part[1023];
 }
 
 // Cell pass of the backward.  FILL = false: scatter with atomics.  FILL = true: write pairs.
-// `cursor` holds, on entry, the start of every texel's segment; phase A advances it, so on
-// exit cursor[t] is the END of texel t's segment (= the start of texel t+1's).
+// `cursor` holds, on entry, the start (within its scan chunk) of every (texel, replica)
+// segment; phase A advances it, so on exit cursor[i] is the END of segment i.
 template <typename T, int VEC, int CPL, bool FILL>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_kernel(
     KParams k, const float *__restrict__ grad_out, const T *__restrict__ depth, const T *__restrict__ feats,
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
-    int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap) {
+    const int *__restrict__ chunk_prefix, int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap) {
     extern __shared__ float4 smem[];
     constexpr int EF4 = FILL ? 4 : 3;
     const int lane = threadIdx.x & (kWave - 1);
@@ -540,7 +625,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
         const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
         if (lane < 16) cnt[lane] = 0;
-        phase_a<EF4, T, FILL ? kModeFill : kModeScatter>(k, Pm, depth, b, q0, lane, lst, cnt, cursor, pair_cap);
+        phase_a<EF4, T, FILL ? kModeFill : kModeScatter>(k, Pm, depth, b, q0, lane, lst, cnt, chunk_prefix, cursor,
+                                                         pair_cap);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
@@ -672,14 +758,16 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
 // sums to d_depth[texel, 0:2]) with plain loads and stores -- the texel is owned by the block.
 template <int VEC>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_kernel(
-    KParams k, const float *__restrict__ grad_out, const int *__restrict__ seg_end,
-    const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth, float *__restrict__ d_feats,
-    int lanes_per_row, int depth_from_pairs) {
+    KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
+    const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
+    float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs) {
     extern __shared__ float4 smem[];
     float *part = reinterpret_cast<float *>(smem);
     const int t = blockIdx.x;
-    const int start = t == 0 ? 0 : seg_end[t - 1];
-    const int end = min(seg_end[t], pair_cap);
+    // the texel's pairs: from the end of the previous texel's last replica to the end of its own
+    const long long first = (long long)t * kReplicas - 1, last = (long long)t * kReplicas + kReplicas - 1;
+    const int start = t == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
+    const int end = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
     if (start >= end) return;      // uniform for the block
     const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
     const int lane = threadIdx.x & (kWave - 1);
@@ -868,6 +956,7 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
     dim3 grid(pl.k.n_blocks), block(kWave * kWavesPerBlock);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
+    prof::Scope timer(prof::kForward, st);
     switch (pl.cpl) {
         case 1: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 1>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out); break;
         case 2: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 2>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out); break;
@@ -878,37 +967,40 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
 
 template <typename T, int VEC, bool FILL>
 int launch_cells(const Plan &pl, const float *go, const void *depth, const void *feats, const float *proj,
-                 float *dd, float *df, int *cursor, Pair *pairs, int cap, hipStream_t st) {
+                 float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap, hipStream_t st) {
     dim3 grid(pl.k.n_blocks), block(kWave * kWavesPerBlock);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
     const size_t lds = FILL ? pl.lds_fill : pl.lds_bwd;
+    prof::Scope timer(FILL ? prof::kBackwardCells : prof::kBackwardScatter, st);
     switch (pl.cpl) {
-        case 1: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, cursor, pairs, cap); break;
-        case 2: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, cursor, pairs, cap); break;
-        default: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, cursor, pairs, cap); break;
+        case 1: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+        case 2: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+        default: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
     }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
 template <bool FILL>
 int dispatch_cells(const fbev_problem *p, const Plan &pl, const float *go, const void *depth, const void *feats,
-                   const float *proj, float *dd, float *df, int *cursor, Pair *pairs, int cap, hipStream_t st) {
+                   const float *proj, float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap,
+                   hipStream_t st) {
     switch (p->in_dtype) {
         case FBEV_F32:
-            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st)
-                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st);
+            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st)
+                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st);
         case FBEV_F16:
-            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st)
-                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st);
+            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st)
+                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st);
         default:
-            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st)
-                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, cursor, pairs, cap, st);
+            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st)
+                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st);
     }
 }
 
 template <typename T>
 int launch_count(const Plan &pl, const void *depth, const float *proj, int *counts, long long total, hipStream_t st) {
+    prof::Scope timer(prof::kCount, st);
     hipLaunchKernelGGL((fbev_count_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, pl.k,
                        static_cast<const T *>(depth), proj, counts, total);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
@@ -922,9 +1014,14 @@ long long sample_count(const fbev_problem *p) {
     return (long long)p->batch * p->grid_y * p->grid_x * p->num_cams * p->grid_z;
 }
 
-// Workspace layout: [texels + 1 int32 segment cursors, padded to 256 bytes][pairs]
+// Workspace layout: [texels * kReplicas int32 segment cursors][chunk prefix sums], padded to
+// 256 bytes, then the pairs.
+long long counter_count(const fbev_problem *p) { return texel_count(p) * kReplicas; }
+long long chunk_count(const fbev_problem *p) {
+    return (counter_count(p) + (1ll << kScanChunkBits) - 1) >> kScanChunkBits;
+}
 size_t ws_index_bytes(const fbev_problem *p) {
-    return (((size_t)texel_count(p) + 1) * sizeof(int) + 255) / 256 * 256;
+    return ((size_t)(counter_count(p) + chunk_count(p) + 1) * sizeof(int) + 255) / 256 * 256;
 }
 
 int check_backward_args(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
@@ -977,7 +1074,7 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
     Plan pl;
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl);
     if (rc != FBEV_OK) return rc;
-    return dispatch_cells<false>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, nullptr, nullptr, 0,
+    return dispatch_cells<false>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, nullptr, nullptr, nullptr, 0,
                                  static_cast<hipStream_t>(stream));
 }
 
@@ -1004,7 +1101,7 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const size_t index_bytes = ws_index_bytes(p);
     if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
     // pair positions are 32-bit: every sample corner must be countable
-    if (4 * sample_count(p) >= (1ll << 31) || texel_count(p) + 1 >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    if (4 * sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
     size_t cap64 = (workspace_bytes - index_bytes) / sizeof(Pair);
     const int cap = cap64 > 0x7fffffffull ? 0x7fffffff : (int)cap64;
     Plan pl;
@@ -1014,9 +1111,14 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     int *cursor = static_cast<int *>(workspace);
     Pair *pairs = reinterpret_cast<Pair *>(static_cast<char *>(workspace) + index_bytes);
     const long long texels = texel_count(p), samples = sample_count(p);
+    const long long counters = counter_count(p), chunks = chunk_count(p);
+    int *chunk_prefix = cursor + counters;
 
-    hipLaunchKernelGGL(fbev_fill_zero_kernel, dim3((unsigned)((texels + 1 + 255) / 256)), dim3(256), 0, st, cursor,
-                       texels + 1);
+    {
+        prof::Scope timer(prof::kZero, st);
+        hipLaunchKernelGGL(fbev_fill_zero_kernel, dim3((unsigned)((counters + 255) / 256)), dim3(256), 0, st, cursor,
+                           counters);
+    }
     if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
     switch (p->in_dtype) {
         case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, samples, st); break;
@@ -1024,9 +1126,19 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
         default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, samples, st); break;
     }
     if (rc != FBEV_OK) return rc;
-    hipLaunchKernelGGL(fbev_scan_kernel, dim3(1), dim3(1024), 0, st, cursor, (int)texels);
+    {
+        prof::Scope timer(prof::kScanChunks, st);
+        hipLaunchKernelGGL(fbev_scan_chunks_kernel, dim3((unsigned)chunks), dim3(1024), 0, st, cursor, counters,
+                           chunk_prefix);
+    }
     if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
-    rc = dispatch_cells<true>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, cursor, pairs, cap, st);
+    {
+        prof::Scope timer(prof::kScanSums, st);
+        hipLaunchKernelGGL(fbev_scan_sums_kernel, dim3(1), dim3(1024), 0, st, chunk_prefix, (int)chunks);
+    }
+    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+    rc = dispatch_cells<true>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, chunk_prefix, cursor, pairs, cap,
+                              st);
     if (rc != FBEV_OK) return rc;
 
     // texel pass: rows of grad_out are fp32, so 128-bit gathers need C % 4 == 0 and aligned rows
@@ -1037,12 +1149,13 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const int nw = (kWave / lpr) * kWavesPerBlock;
     const size_t lds = (size_t)nw * (lpr * vec + 2) * sizeof(float);
     const int from_pairs = (d_depth != nullptr && p->depth_distribution != FBEV_CATEGORICAL) ? 1 : 0;
+    prof::Scope timer(prof::kBackwardTexel, st);
     if (vec4)
         hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels), dim3(kWave * kWavesPerBlock), lds,
-                           st, pl.k, grad_out, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
+                           st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
     else
         hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels), dim3(kWave * kWavesPerBlock), lds,
-                           st, pl.k, grad_out, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
+                           st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
@@ -1061,6 +1174,7 @@ int fbev_sample_geometry(const fbev_problem *p, const float *proj, uint8_t *mask
     const long long total = (long long)p->batch * p->grid_y * p->grid_x * p->num_cams * p->grid_z;
     const long long blocks = (total + 255) / 256;
     if (blocks >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    prof::Scope timer(prof::kGeometry, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(fbev_geometry_kernel, dim3((unsigned)blocks), dim3(256), 0,
                        static_cast<hipStream_t>(stream), pl.k, proj, mask, idx, frac, total);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
@@ -1089,6 +1203,37 @@ const char *fbev_status_string(int status) {
         case FBEV_ERR_LAUNCH: return "HIP reported a kernel launch error";
         default: return "unknown status";
     }
+}
+
+int fbev_profile_enable(int on) {
+    std::lock_guard<std::mutex> g(prof::mu);
+    for (auto &r : prof::recs) { (void)hipEventDestroy(r.a); (void)hipEventDestroy(r.b); }
+    prof::recs.clear();
+    prof::enabled.store(on != 0);
+    return FBEV_OK;
+}
+
+int fbev_profile_kernel_count(void) { return prof::kNum; }
+
+const char *fbev_profile_kernel_name(int kernel) {
+    return (kernel >= 0 && kernel < prof::kNum) ? prof::kNames[kernel] : "";
+}
+
+int fbev_profile_collect(double *total_ms, int64_t *calls) {
+    if (!total_ms || !calls) return FBEV_ERR_NULL;
+    std::lock_guard<std::mutex> g(prof::mu);
+    for (int i = 0; i < prof::kNum; ++i) { total_ms[i] = 0.0; calls[i] = 0; }
+    int rc = FBEV_OK;
+    for (auto &r : prof::recs) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(r.b) != hipSuccess || hipEventElapsedTime(&ms, r.a, r.b) != hipSuccess) rc = FBEV_ERR_LAUNCH;
+        total_ms[r.kid] += ms;
+        calls[r.kid] += 1;
+        (void)hipEventDestroy(r.a);
+        (void)hipEventDestroy(r.b);
+    }
+    prof::recs.clear();
+    return rc;
 }
 
 int fbev_abi_version(void) { return FBEV_ABI_VERSION; }

@@ -135,6 +135,19 @@ int fbev_sample_geometry(const fbev_problem *p, const float *proj, uint8_t *mask
 /* Compulsory bytes moved by one call: every operand tensor once (backward != 0 selects the backward). */
 uint64_t fbev_algorithmic_bytes(const fbev_problem *p, int backward);
 
+/*
+ * Opt-in per-kernel timing for benchmarks.  While enabled, every kernel this library launches
+ * is bracketed by a pair of HIP events on the launch stream (so enabling it makes calls
+ * allocate events).  fbev_profile_collect waits for all recorded events, writes the summed
+ * duration (ms) and launch count of each of the fbev_profile_kernel_count() kernels, and
+ * clears the record.  No counterpart in the reference, which times whole calls with
+ * time.perf_counter (tools/utils/benchmark_utils.py:44-69).
+ */
+int fbev_profile_enable(int on);
+int fbev_profile_kernel_count(void);
+const char *fbev_profile_kernel_name(int kernel);
+int fbev_profile_collect(double *total_ms, int64_t *calls);
+
 const char *fbev_status_string(int status);
 int fbev_abi_version(void);
 size_t fbev_problem_size(void);

@@ -1,0 +1,242 @@
+"""CPU-side checks: the C-ABI library loads and exports what include/flashbev_hip.h declares,
+argument validation returns the documented status codes without touching a GPU, the Python
+operator marshals its arguments like the reference's (flashbev/flashbevpool/flash_bevpool.py:22-136),
+and the workload generator reproduces the byte counts the benchmark prices against."""
+import ctypes
+import os
+import re
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import flashbev_amd
+from flashbev_amd import _build, capi
+from flashbev_amd.flash_bevpool import FlashBEVPool, flash_bevpool, voxel_geometry
+from flashbev_amd.workloads import WORKLOADS, algorithmic_bytes, make_inputs
+
+op_module = sys.modules["flashbev_amd.flash_bevpool"]   # the package attribute of that name is the function
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "flashbev_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fbev_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.load()
+    names = header_functions()
+    assert len(names) >= 10
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in flashbev_hip.h but not exported"
+    assert sorted(capi.EXPORTS) == names
+    assert lib.fbev_abi_version() == 1
+    assert lib.fbev_problem_size() == ctypes.sizeof(capi.FbevProblem)
+
+
+def test_header_struct_matches_binding():
+    text = open(os.path.join(ROOT, "include", "flashbev_hip.h")).read()
+    body = re.search(r"typedef struct fbev_problem \{(.*?)\} fbev_problem;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = re.findall(r"(?:int32_t|float)\s+([a-z_]+)(?:\[\d\])?;", body)
+    assert fields == [f[0] for f in capi.FbevProblem._fields_]
+
+
+def good_problem(**kw):
+    args = dict(batch=1, num_cams=2, feat_hw=(4, 6), channels=8, image_hw=(64, 96), grid_size=(5, 5, 2),
+                voxel_min=(0.0, -5.0, -2.0), voxel_size=(2.0, 2.0, 2.0))
+    args.update(kw)
+    return capi.make_problem(**args)
+
+
+def test_validation_status_codes_without_gpu():
+    """Bad arguments are rejected before any HIP call, so this runs without a GPU."""
+    ok = good_problem()
+    assert capi.forward(ok, 0, 0, 0, 0) == -1 and "NULL" in capi.status_string(-1)
+    assert capi.forward(good_problem(channels=0), 16, 16, 16, 16) == -2
+    assert capi.forward(good_problem(grid_size=(5, 0, 2)), 16, 16, 16, 16) == -2
+    assert capi.forward(good_problem(proj_stride=9), 16, 16, 16, 16) == -2
+    assert capi.forward(good_problem(in_dtype=7), 16, 16, 16, 16) == -3
+    assert capi.forward(good_problem(depth_distribution=3), 16, 16, 16, 16) == -3
+    assert capi.forward(good_problem(depth_bins=5), 16, 16, 16, 16) == -2          # parametric needs 2
+    assert capi.forward(good_problem(depth_distribution=2, depth_bins=16, depth_range=(1.0, 0.0)), 16, 16, 16, 16) == -2
+    assert capi.forward(ok, 16, 16, 18, 16) == -5                                   # proj not 4-byte aligned
+    assert capi.forward(good_problem(in_dtype=capi.FBEV_F16), 17, 16, 16, 16) == -5
+    assert capi.forward(good_problem(batch=1 << 20, num_cams=64, feat_hw=(64, 64)), 16, 16, 16, 16) == -4
+    assert capi.forward(good_problem(num_cams=64, grid_size=(5, 5, 64)), 16, 16, 16, 16) == -4   # LDS lists
+    assert capi.backward(ok, 0, 16, 16, 16, 16, 16) == -1
+    assert capi.backward(ok, 16, 16, 16, 16, None, None) == 0                      # nothing asked for
+    assert capi.backward_gather(ok, 16, 16, 16, 16, 16, 16, 0, 0) == -1            # no workspace
+    assert capi.backward_gather(ok, 16, 16, 16, 16, 16, 16, 32, 8) == -2           # workspace too small
+    assert capi.sample_geometry(ok, 0, 16, 16, 16) == -1
+    for rc in range(-6, 1):
+        assert capi.status_string(rc) != "unknown status"
+    assert capi.status_string(-99) == "unknown status"
+
+
+def test_workspace_and_byte_helpers():
+    p = good_problem()
+    assert capi.backward_max_pairs(p) == 4 * 1 * 5 * 5 * 2 * 2
+    w0 = capi.backward_workspace_bytes(p, 0)
+    assert w0 > 0 and w0 % 256 == 0
+    assert capi.backward_workspace_bytes(p, 100) == w0 + 1600
+    # compulsory bytes: every operand once
+    texels = 1 * 2 * 4 * 6
+    fwd = texels * 8 * 4 + texels * 2 * 4 + 2 * 48 + 5 * 5 * 8 * 4
+    assert capi.algorithmic_bytes(p, False) == fwd
+    assert capi.algorithmic_bytes(p, True) == fwd + texels * 8 * 4 + texels * 2 * 4
+
+
+@pytest.mark.parametrize("name,model,backward,expected", [
+    ("cfg1_tiny", "categorical", False, 99376), ("cfg1_tiny", "parametric", False, 78256),
+    ("cfg2_surround", "categorical", False, 7591712), ("cfg2_surround", "parametric", False, 6628640),
+    ("cfg3_zsweep", "categorical", False, 15148832), ("cfg3_zsweep", "parametric", False, 14185760),
+    ("cfg4_hires", "categorical", False, 167470208), ("cfg4_hires", "parametric", False, 151790720),
+    ("cfg5_train", "categorical", False, 348971264), ("cfg5_train", "parametric", False, 345118976),
+])
+def test_workload_bytes_match_the_measurement_plan(name, model, backward, expected):
+    assert algorithmic_bytes(WORKLOADS[name], model, backward) == expected
+
+
+def test_fwd_bwd_bytes_match_the_measurement_plan():
+    w = WORKLOADS["cfg2_surround"]
+    assert algorithmic_bytes(w, "parametric", False) + algorithmic_bytes(w, "parametric", True) == 14642752
+    assert algorithmic_bytes(w, "categorical", False) + algorithmic_bytes(w, "categorical", True) == 17531968
+    w = WORKLOADS["cfg5_train"]
+    assert algorithmic_bytes(w, "parametric", False) + algorithmic_bytes(w, "parametric", True) == 725111296
+
+
+def test_workload_generator_shapes_and_seeding():
+    w = WORKLOADS["cfg2_surround"]
+    a = make_inputs(w, "parametric")
+    b = make_inputs(w, "parametric")
+    assert torch.equal(a["image_feats"], b["image_feats"]) and torch.equal(a["projection_matrices"], b["projection_matrices"])
+    assert a["image_feats"].shape == (1, 6, 16, 44, 80) and a["depth_params"].shape == (1, 6, 16, 44, 2)
+    assert a["projection_matrices"].shape == (1, 6, 3, 4) and a["grad_out"].shape == (1, 128, 128, 80)
+    assert (a["depth_params"][..., 1] >= 0.5).all() and (a["depth_params"][..., 0] >= 5.0).all()
+    c = make_inputs(w, "categorical")
+    assert c["depth_params"].shape[-1] == 59 and torch.allclose(c["depth_params"].sum(-1), torch.ones(1, 6, 16, 44))
+    assert make_inputs(WORKLOADS["cfg4_hires"].with_z(2), "parametric")["image_feats"].dtype == torch.bfloat16
+    # per-batch jitter differs
+    p4 = make_inputs(WORKLOADS["cfg4_hires"].with_z(2), "parametric")["projection_matrices"]
+    assert not torch.equal(p4[0], p4[1])
+
+
+def test_voxel_geometry_is_fp32_arithmetic():
+    vmin, vsize = voxel_geometry((-51.2, 51.2, -51.2, 51.2, -5.0, 3.0), (200, 200, 12))
+    r = np.float32([-51.2, 51.2, -5.0, 3.0])
+    assert vsize[0] == float((r[1] - r[0]) / np.float32(200))
+    assert vsize[2] == float((r[3] - r[2]) / np.float32(12))
+    assert vmin == [float(r[0]), float(r[0]), float(r[2])]
+
+
+class FakeExt:
+    """Stands in for flashbevpool_ext so that the operator's host logic runs without a GPU."""
+
+    def __init__(self):
+        self.fwd = self.bwd = None
+
+    def flash_bevpool_forward(self, *a):
+        self.fwd = a
+        a[12].fill_(1.0)
+
+    def flash_bevpool_backward(self, *a):
+        self.bwd = a
+        if a[8] is not None:
+            a[8].add_(2.0)
+        if a[9] is not None:
+            a[9].add_(3.0)
+
+
+@pytest.fixture
+def fake_ext(monkeypatch):
+    ext = FakeExt()
+    monkeypatch.setattr(op_module, "load_ext", lambda: ext)
+
+    # the operator insists on a GPU tensor; let CPU tensors pass for this host-logic test
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+    return ext
+
+
+def test_operator_marshalling_matches_reference_order(fake_ext):
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    f = x["image_feats"].clone().requires_grad_(True)
+    d = x["depth_params"].clone().requires_grad_(True)
+    # 14 positional arguments, exactly like the reference's apply()
+    out = FlashBEVPool.apply(d, f, x["projection_matrices"], x["feature_size"], x["image_size"], x["roi_range"],
+                             x["grid_size"], 1, True, True, False, False, 1e-6, 0.0)
+    a = fake_ext.fwd
+    assert out.shape == (1, 32, 32, 16) and out.dtype == torch.float32
+    assert a[0].shape == d.shape and a[1].shape == f.shape           # depth first, then feats
+    vmin, vsize = voxel_geometry(w.roi_range, w.grid_size)
+    assert list(a[6:9]) == vsize and list(a[9:12]) == vmin
+    assert a[13] == out.numel() and a[14] == 1                        # total_threads, depth_distribution
+    assert a[19] == pytest.approx(1e-6) and a[20] == 0.0
+    out.backward(torch.ones_like(out))                                # 16 returned grads, 14 inputs: accepted
+    b = fake_ext.bwd
+    assert b[6].tolist() == pytest.approx(list(w.roi_range)) and b[7].tolist() == list(w.grid_size)
+    assert torch.all(d.grad == 2.0) and torch.all(f.grad == 3.0)
+    assert b[8].dtype == torch.float32 and b[9].dtype == torch.float32
+
+
+def test_wrapper_puts_feats_first_and_skips_unneeded_grads(fake_ext):
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    f = x["image_feats"].clone().requires_grad_(True)
+    out = flash_bevpool(f, x["depth_params"], x["projection_matrices"], x["feature_size"], [128, 352],
+                        list(w.roi_range), list(w.grid_size), depth_distribution=0)
+    out.sum().backward()
+    assert fake_ext.bwd[8] is None and fake_ext.bwd[9] is not None     # depth grad not requested
+    assert f.grad is not None
+
+
+def test_half_inputs_are_not_upcast_and_mixed_dtypes_are(fake_ext):
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    flash_bevpool(x["image_feats"].half(), x["depth_params"].half(), x["projection_matrices"], x["feature_size"],
+                  x["image_size"], x["roi_range"], x["grid_size"])
+    assert fake_ext.fwd[0].dtype == torch.float16 and fake_ext.fwd[1].dtype == torch.float16
+    flash_bevpool(x["image_feats"].half(), x["depth_params"], x["projection_matrices"], x["feature_size"],
+                  x["image_size"], x["roi_range"], x["grid_size"])
+    assert fake_ext.fwd[0].dtype == torch.float32 and fake_ext.fwd[1].dtype == torch.float32
+
+
+def test_operator_argument_errors(fake_ext):
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    base = (x["image_feats"], x["depth_params"], x["projection_matrices"], x["feature_size"], x["image_size"],
+            x["roi_range"], x["grid_size"])
+    with pytest.raises(ValueError, match="depth_distribution"):
+        flash_bevpool(*base, depth_distribution=5)
+    with pytest.raises(ValueError, match="depth_range"):
+        flash_bevpool(*base, depth_distribution=2)
+    with pytest.raises(ValueError, match="reduction"):
+        flash_bevpool(*base, reduction="max")
+    with pytest.raises(ValueError, match="grid_size"):
+        flash_bevpool(*base[:6], [32, 32])
+
+
+def test_operator_refuses_cpu_tensors():
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        flash_bevpool(x["image_feats"], x["depth_params"], x["projection_matrices"], x["feature_size"],
+                      x["image_size"], x["roi_range"], x["grid_size"])
+
+
+def test_package_exports():
+    assert set(flashbev_amd.__all__) >= {"FlashBEVPool", "flash_bevpool", "create_projection_matrix"}
+    assert os.path.exists(_build.HIP_LIB) and os.path.exists(_build.EXT_LIB)
+
+
+def test_product_never_imports_the_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "flashbev_amd")):
+        for fn in files:
+            if fn.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, fn)).read()
+                assert "oracle" not in text.replace("oracle-free", ""), f"{fn} mentions the oracle"
