@@ -3,9 +3,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--table]
 
 One step = one forward plus one backward pass of the operator over one batch of seeded
-synthetic input that is already resident in HBM: forward kernel, zero-fill of the two
-gradient buffers, backward kernel, all queued on PyTorch's current stream through the
-extension module.  The default workload is the 6-camera 128x128x8 fp32 configuration
+synthetic input that is already resident in HBM: the forward kernel (which also records the
+per-cell sample counts) and the backward kernels (whose first launch zero-fills the two
+gradient buffers), all queued on PyTorch's current stream through the extension module.  The default workload is the 6-camera 128x128x8 fp32 configuration
 (``cfg2_surround``) with the reference benchmark's depth model (per-pixel Laplace
 parameters, tools/config/config.yaml:29).  The single JSON line printed on stdout carries
   value / ms_per_step   forward+backward latency per step (ms)
@@ -56,8 +56,9 @@ class Runner:
         B, N, H, W, C = x["image_feats"].shape
         gx, gy, gz = w.grid_size
         self.out = torch.empty((B, gy, gx, C), dtype=torch.float32, device=device)
-        self.d_depth = torch.zeros(x["depth_params"].shape, dtype=torch.float32, device=device)
-        self.d_feats = torch.zeros(x["image_feats"].shape, dtype=torch.float32, device=device)
+        self.d_depth = torch.empty(x["depth_params"].shape, dtype=torch.float32, device=device)
+        self.d_feats = torch.empty(x["image_feats"].shape, dtype=torch.float32, device=device)
+        self.counts = torch.empty((B, gy, gx), dtype=torch.float32, device=device)
         self.vmin, self.vsize = voxel_geometry(w.roi_range, w.grid_size)
         self.eps, self.thr = 1e-6, 1e-6
 
@@ -67,18 +68,15 @@ class Runner:
             x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"], x["image_size"],
             x["grid_size"], self.vsize[0], self.vsize[1], self.vsize[2], self.vmin[0], self.vmin[1],
             self.vmin[2], self.out, self.out.numel(), self.dist, True, True, False, False, self.eps, self.thr,
-            w.depth_range[0], w.depth_range[1], 0)
-
-    def zero_grads(self):
-        self.d_depth.zero_()
-        self.d_feats.zero_()
+            w.depth_range[0], w.depth_range[1], 0, self.counts)
 
     def backward(self):
         x, w = self.x, self.w
         self.ext.flash_bevpool_backward(
             x["grad_out"], x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
             x["image_size"], x["roi_range"], x["grid_size"], self.d_depth, self.d_feats, self.out.numel(),
-            self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0, self.backward_mode, -1)
+            self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0, self.backward_mode, -1,
+            self.counts, False)
 
 
 def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
@@ -86,7 +84,6 @@ def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
     for _ in range(warmup):
         r.forward()
         if with_backward:
-            r.zero_grads()
             r.backward()
     torch.cuda.synchronize()
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
@@ -97,7 +94,6 @@ def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
         r.forward()
         ev[i][1].record()
         if with_backward:
-            r.zero_grads()
             ev[i][2].record()
             r.backward()
             ev[i][3].record()
@@ -114,7 +110,6 @@ def profile_steps(r: Runner, steps: int):
     try:
         for _ in range(steps):
             r.forward()
-            r.zero_grads()
             r.backward()
         torch.cuda.synchronize()
         got = capi.profile_collect()
@@ -200,8 +195,8 @@ def main():
     ap.add_argument("--depth", default="laplace", choices=sorted(DIST_OF))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--table", action="store_true")
-    ap.add_argument("--backward-mode", type=int, default=0, choices=(0, 1, 2),
-                    help="0/2 inverse-map gather (default), 1 atomic scatter")
+    ap.add_argument("--backward-mode", type=int, default=0, choices=(0, 1, 2, 3),
+                    help="0 auto (default), 1 atomic scatter, 2 inverse-map gather, 3 column owner")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="only run a device-to-device copy of this many MiB (counter calibration)")
     args = ap.parse_args()
@@ -245,8 +240,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": w.name, "depth_model": args.depth, "batch": w.batch, "cams": w.num_cams,
                    "channels": w.channels, "feat_hw": list(w.feat_hw), "grid": list(w.grid_size),
-                   "backward": {0: "inverse-map gather", 1: "atomic scatter", 2: "inverse-map gather"}[args.backward_mode],
-                   "step": "forward kernel + zero-fill of both gradient buffers + backward kernels"},
+                   "backward": {0: "auto", 1: "atomic scatter", 2: "inverse-map gather", 3: "column owner"}[args.backward_mode],
+                   "step": "forward kernel + backward kernels (gradient zero-fill folded into the first)"},
         "fwd_call_ms": stats(fwd), "bwd_call_ms": stats(bwd),
         "effective_GBps_fwd_bwd": (fb + bb) / ms / 1e6,
         "frac_hbm_fwd_bwd": (fb + bb) / ms / 1e6 / HBM_PEAK_GBS,

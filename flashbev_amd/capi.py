@@ -15,7 +15,8 @@ FBEV_F32, FBEV_F16, FBEV_BF16 = 0, 1, 2
 FBEV_GAUSSIAN, FBEV_LAPLACE, FBEV_CATEGORICAL = 0, 1, 2
 FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
-EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_max_pairs",
+EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_columns",
+           "fbev_backward_columns_workspace_bytes", "fbev_backward_max_pairs",
            "fbev_backward_workspace_bytes", "fbev_sample_geometry", "fbev_algorithmic_bytes",
            "fbev_profile_enable", "fbev_profile_kernel_count", "fbev_profile_kernel_name",
            "fbev_profile_collect", "fbev_status_string", "fbev_abi_version", "fbev_problem_size")
@@ -43,12 +44,16 @@ def load() -> ctypes.CDLL:
     if _lib is None:
         lib = ctypes.CDLL(_build.HIP_LIB)
         vp, pp = ctypes.c_void_p, ctypes.POINTER(FbevProblem)
-        lib.fbev_forward.argtypes = [pp, vp, vp, vp, vp, vp]
+        lib.fbev_forward.argtypes = [pp, vp, vp, vp, vp, vp, vp]
         lib.fbev_forward.restype = ctypes.c_int
-        lib.fbev_backward.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp]
+        lib.fbev_backward.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp]
         lib.fbev_backward.restype = ctypes.c_int
-        lib.fbev_backward_gather.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp]
+        lib.fbev_backward_gather.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp, ctypes.c_size_t, vp]
         lib.fbev_backward_gather.restype = ctypes.c_int
+        lib.fbev_backward_columns.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp, ctypes.c_size_t, vp]
+        lib.fbev_backward_columns.restype = ctypes.c_int
+        lib.fbev_backward_columns_workspace_bytes.argtypes = [pp]
+        lib.fbev_backward_columns_workspace_bytes.restype = ctypes.c_size_t
         lib.fbev_backward_max_pairs.argtypes = [pp]
         lib.fbev_backward_max_pairs.restype = ctypes.c_uint64
         lib.fbev_backward_workspace_bytes.argtypes = [pp, ctypes.c_uint64]
@@ -112,23 +117,37 @@ def _p(ptr: Optional[int]):
 
 
 def forward(p: FbevProblem, depth_ptr: int, feats_ptr: int, proj_ptr: int, out_ptr: int,
-            stream: int = 0) -> int:
+            stream: int = 0, count_ptr: Optional[int] = None) -> int:
     return load().fbev_forward(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(proj_ptr), _p(out_ptr),
-                               _p(stream))
+                               _p(count_ptr), _p(stream))
 
 
 def backward(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
-             d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], stream: int = 0) -> int:
+             d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], stream: int = 0,
+             accumulate: bool = True) -> int:
     return load().fbev_backward(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
-                                _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), _p(stream))
+                                _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), int(bool(accumulate)), _p(stream))
 
 
 def backward_gather(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
                     d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], workspace_ptr: int,
-                    workspace_bytes: int, stream: int = 0) -> int:
+                    workspace_bytes: int, stream: int = 0, accumulate: bool = True) -> int:
     return load().fbev_backward_gather(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
-                                       _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), _p(workspace_ptr),
-                                       ctypes.c_size_t(int(workspace_bytes)), _p(stream))
+                                       _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), int(bool(accumulate)),
+                                       _p(workspace_ptr), ctypes.c_size_t(int(workspace_bytes)), _p(stream))
+
+
+def backward_columns(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
+                     count_ptr: Optional[int], d_depth_ptr: Optional[int], d_feats_ptr: Optional[int],
+                     accumulate: bool, workspace_ptr: Optional[int], workspace_bytes: int, stream: int = 0) -> int:
+    return load().fbev_backward_columns(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
+                                        _p(proj_ptr), _p(count_ptr), _p(d_depth_ptr), _p(d_feats_ptr),
+                                        int(bool(accumulate)), _p(workspace_ptr),
+                                        ctypes.c_size_t(int(workspace_bytes)), _p(stream))
+
+
+def backward_columns_workspace_bytes(p: FbevProblem) -> int:
+    return int(load().fbev_backward_columns_workspace_bytes(ctypes.byref(p)))
 
 
 def backward_max_pairs(p: FbevProblem) -> int:

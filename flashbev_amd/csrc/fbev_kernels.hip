@@ -39,11 +39,12 @@ namespace {
 // call count per kernel.  Disabled (the default) it costs one relaxed atomic load per launch.
 namespace prof {
 enum Kid { kForward, kBackwardScatter, kZero, kCount, kScanChunks, kScanSums, kBackwardCells, kBackwardTexel,
-           kGeometry, kNum };
+           kGeometry, kBackwardColumn, kCellCount, kNum };
 const char *const kNames[kNum] = {"fbev_forward_kernel", "fbev_backward_cells_kernel<scatter>",
                                   "fbev_fill_zero_kernel", "fbev_count_kernel", "fbev_scan_chunks_kernel",
                                   "fbev_scan_sums_kernel", "fbev_backward_cells_kernel<fill>",
-                                  "fbev_backward_texel_kernel", "fbev_geometry_kernel"};
+                                  "fbev_backward_texel_kernel", "fbev_geometry_kernel",
+                                  "fbev_backward_column_kernel", "fbev_forward_kernel<count only>"};
 struct Rec { hipEvent_t a, b; int kid; };
 std::atomic<bool> enabled{false};
 std::mutex mu;
@@ -371,7 +372,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const
 template <typename T, int VEC, int CPL>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     KParams k, const T *__restrict__ depth, const T *__restrict__ feats, const float *__restrict__ proj,
-    float *__restrict__ out) {
+    float *__restrict__ out, float *__restrict__ count_out) {
     extern __shared__ float4 smem[];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -409,8 +410,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
         bool mine = carrier && cell_of(k, q0 + slot, ix, iy);
         const int n = mine ? cnt[slot] : 0;
         const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * 2;
+        // the number of samples that enter the mean; the backward pass can reuse it
+        if (count_out != nullptr && mine && lis == 0) count_out[((size_t)b * k.gy + iy) * k.gx + ix] = (float)n;
         float *o = out + (((size_t)b * k.gy + iy) * k.gx + ix) * k.C;
-        for (int c0 = 0; c0 < k.C; c0 += span) {
+        for (int c0 = 0; out != nullptr && c0 < k.C; c0 += span) {
             float acc[CPL][VEC];
 #pragma unroll
             for (int j = 0; j < CPL; ++j)
@@ -487,9 +490,15 @@ struct Pair {      // 16 bytes
     float da, db;  // this sample's contribution to d_depth[texel, 0] and [texel, 1] (parametric models)
 };
 
-__global__ __launch_bounds__(256) void fbev_fill_zero_kernel(int *p, long long n) {
+// Zero up to three regions of 32-bit words in one launch (segment counters and, when the
+// library is asked to, the two gradient buffers).  A kernel rather than hipMemsetAsync, so the
+// call can be captured in a HIP graph.
+__global__ __launch_bounds__(256) void fbev_fill_zero_kernel(int *a, long long na, int *b, long long nb, int *c,
+                                                             long long nc) {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0;
+    if (i < na) a[i] = 0;
+    else if (i < na + nb) b[i - na] = 0;
+    else if (i < na + nb + nc) c[i - na - nb] = 0;
 }
 
 // One thread per (cell, camera, height) sample: count, per texel, the sample corners that
@@ -752,10 +761,15 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     }
 }
 
-// Texel pass of the inverse-map backward: one block per texel.  Its 4 * (64 / lanes_per_row)
-// workers stride over the texel's pairs, each gathering grad_out rows with 128-bit loads;
-// partial rows meet in LDS and the block adds the sum to d_feats[texel, :] (and the depth
-// sums to d_depth[texel, 0:2]) with plain loads and stores -- the texel is owned by the block.
+// Texel pass of the inverse-map backward.  A texel's pairs are handled by one block, or, when
+// there are more than kTexelPart of them (the texels on the horizon collect thousands), by up
+// to kTexelSplit blocks (blockIdx.y) that each take an equal share.  A block's
+// 4 * (64 / lanes_per_row) workers stride over its pairs, each gathering grad_out rows with
+// 128-bit loads; partial rows meet in LDS.  A texel handled by one block is updated with plain
+// loads and stores; the shares of a split texel are combined with fp32 atomics (at most
+// kTexelSplit per address).
+constexpr int kTexelSplit = 8;
+constexpr int kTexelPart = 128;
 template <int VEC>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_kernel(
     KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
@@ -766,9 +780,19 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
     const int t = blockIdx.x;
     // the texel's pairs: from the end of the previous texel's last replica to the end of its own
     const long long first = (long long)t * kReplicas - 1, last = (long long)t * kReplicas + kReplicas - 1;
-    const int start = t == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
-    const int end = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
+    int start = t == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
+    int end = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
     if (start >= end) return;      // uniform for the block
+    const int n_all = end - start;
+    const int n_parts = min(kTexelSplit, (n_all + kTexelPart - 1) / kTexelPart);
+    if ((int)blockIdx.y >= n_parts) return;
+    {
+        const int s0 = start + (int)(((long long)n_all * blockIdx.y) / n_parts);
+        const int s1 = start + (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
+        start = s0;
+        end = s1;
+    }
+    const bool shared_texel = n_parts > 1;
     const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -823,14 +847,477 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
         for (int c = threadIdx.x; c < span && c0 + c < k.C; c += blockDim.x) {
             float sum = 0.0f;
             for (int w = 0; w < nw; ++w) sum += part[w * stride + c];
-            if (d_feats != nullptr) d_feats[(size_t)t * k.C + c0 + c] += sum;
+            if (d_feats != nullptr) {
+                float *dst = d_feats + (size_t)t * k.C + c0 + c;
+                if (shared_texel) atomic_add_f32(dst, sum);
+                else *dst += sum;
+            }
         }
         if (c0 == 0 && depth_from_pairs && threadIdx.x < 2) {
             float sum = 0.0f;
             for (int w = 0; w < nw; ++w) sum += part[w * stride + span + threadIdx.x];
-            d_depth[(size_t)t * 2 + threadIdx.x] += sum;
+            float *dst = d_depth + (size_t)t * 2 + threadIdx.x;
+            if (shared_texel) atomic_add_f32(dst, sum);
+            else *dst += sum;
         }
     }
+}
+
+// ---------------------------------------------------------------- backward, column owner
+// One block owns one column (b, camera, u) of the feature map: all H texels of that column,
+// all channels.  Every sample that touches the column lies in a thin wedge of the BEV grid.
+//   (1) cull   keep the 8x8-cell tiles, then the cells, whose projected u-range can reach the
+//              column.  For a perspective map u = U/D is monotone along every segment in
+//              front of the camera, so its extremes over a box (tile footprint x height range)
+//              or a segment (one cell, all heights) sit at the vertices / end points; whatever
+//              comes near the camera plane is kept unconditionally.  Culling only discards:
+//              every kept sample is decided by the canonical arithmetic.
+//   (2) sample re-project the kept cells' samples; those with a corner in the column become
+//              32-byte entries in LDS.
+//   (3) G      per entry, <grad_out / count, sampled feature> (needed by the depth gradient).
+//   (4) rows   bucket the entries' row contributions by row (LDS integer atomics), share the
+//              slots of the block among the rows in proportion to their length, let every slot
+//              gather grad_out rows into registers, and add the partial rows in a fixed order.
+//   (5) store  every d_feats / d_depth element of the column is written by this block alone.
+// No floating-point atomics on the feature gradient (LDS float atomics cost about two clocks
+// per lane on this machine, global ones serialise per address), no workspace, one launch.
+// The per-cell sample count that the mean divides by comes from the forward pass or from a
+// recount launch.
+constexpr int kColThreads = 512;
+constexpr int kColWaves = kColThreads / kWave;
+constexpr int kColCells = 2048;          // candidate cells per batch (32 tiles)
+constexpr int kColEntries = 1024;        // entries buffered before they are consumed
+constexpr int kColMaxRows = 256;
+constexpr float kCullMargin = 0.05f;     // texels; fp32 error of u is < 1e-2 once D > kCullNear
+constexpr float kCullNear = 0.25f;       // metres in front of the camera plane
+
+struct ColParams {
+    int n_tiles;          // tiles per batch element
+    int lanes_per_slot;   // lanes that carry one grad_out row
+    int slots;            // rows in flight per wavefront
+    int part_stride;      // floats per slot in the partial-row buffer (C + 2, padded)
+    int accumulate;       // add to the gradient buffers instead of overwriting them
+    int n_blocks;
+};
+
+struct ColLds {
+    float *Pm;
+    volatile int *ctrl;    // 0: tiles kept, 1: cells kept, 2: entries
+    int *tiles, *cells, *contrib, *rowcnt, *rowstart, *rowfill, *wk_row, *wk_first, *wk_n;
+    float4 *entries;
+    float *G, *part;
+};
+
+// Append `keep` lanes' values to a list with one LDS atomic per wavefront.
+__device__ __forceinline__ int wave_append(volatile int *counter, bool keep, int lane) {
+    const unsigned long long m = __ballot(keep);
+    int base = 0;
+    if (lane == 0 && m != 0ull) base = atomicAdd(const_cast<int *>(counter), __popcll(m));
+    base = __shfl(base, 0, kWave);
+    return base + __popcll(m & lanemask_lt(lane));
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void column_consume(const KParams &k, const ColParams &cp, const ColLds &L, int n_ent,
+                                               int u, int rowbase, bool first_flush,
+                                               const float *__restrict__ grad_out, const T *__restrict__ feats,
+                                               float *__restrict__ d_depth, float *__restrict__ d_feats) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int slot = lane / cp.lanes_per_slot, lis = lane - slot * cp.lanes_per_slot;
+    const bool carrier = slot < cp.slots;
+    const int worker = wave * cp.slots + slot, n_workers = kColWaves * cp.slots;
+    const int span = cp.lanes_per_slot * VEC;
+    const bool need_f = d_feats != nullptr, need_d = d_depth != nullptr;
+    const bool parametric = k.dist != FBEV_CATEGORICAL;
+    const int Dd = k.Dd;
+
+    // ---- (3) G per entry.  UNR entries per slot could be kept in flight; measured, a deeper
+    // pipeline costs more in occupancy than it hides in latency, so it stays at one.
+    if (need_d) {
+        constexpr int UNR = 1;
+        const int iters = (n_ent + n_workers - 1) / n_workers;
+        for (int it = 0; it < iters; it += UNR) {
+            bool live[UNR];
+            float G[UNR], w00[UNR], w01[UNR], w10[UNR], w11[UNR];
+            const float *go[UNR];
+            const T *p00[UNR], *p01[UNR], *p10[UNR], *p11[UNR];
+#pragma unroll
+            for (int q = 0; q < UNR; ++q) {
+                const int e = (it + q) * n_workers + worker;
+                live[q] = carrier && it + q < iters && e < n_ent;
+                G[q] = 0.0f;
+                const float4 e0 = L.entries[2 * (live[q] ? e : 0)];
+                const int word = __float_as_int(e0.x);
+                const bool c0 = (word >> 30) & 1, c1 = (word >> 31) & 1;
+                const int v0 = __float_as_int(e0.y) & 0xffff, v1 = (__float_as_int(e0.y) >> 16) & 0xffff;
+                const float du = e0.z, dv = e0.w;
+                w00[q] = (1.0f - du) * (1.0f - dv); w01[q] = (1.0f - du) * dv;
+                w10[q] = du * (1.0f - dv); w11[q] = du * dv;
+                const int u0 = c0 ? u : u - 1;
+                const int u1 = c0 ? (c1 ? u : min(u + 1, k.W - 1)) : u;
+                go[q] = grad_out + (size_t)(word & 0x3fffffff) * k.C;
+                p00[q] = feats + (size_t)((rowbase + v0) * k.W + u0) * k.C;
+                p01[q] = feats + (size_t)((rowbase + v1) * k.W + u0) * k.C;
+                p10[q] = feats + (size_t)((rowbase + v0) * k.W + u1) * k.C;
+                p11[q] = feats + (size_t)((rowbase + v1) * k.W + u1) * k.C;
+            }
+            for (int ch = lis * VEC; ch < k.C; ch += span) {
+                float g[UNR][VEC], f00[UNR][VEC], f01[UNR][VEC], f10[UNR][VEC], f11[UNR][VEC];
+#pragma unroll
+                for (int q = 0; q < UNR; ++q) {
+                    if (live[q]) {
+                        VecLoad<float, VEC == 1 ? 1 : 4>::ld(go[q] + ch, *reinterpret_cast<float(*)[VEC == 1 ? 1 : 4]>(&g[q][0]));
+                        if (VEC == 8) VecLoad<float, 4>::ld(go[q] + ch + 4, *reinterpret_cast<float(*)[4]>(&g[q][VEC == 8 ? 4 : 0]));
+                        VecLoad<T, VEC>::ld(p00[q] + ch, f00[q]);
+                        VecLoad<T, VEC>::ld(p01[q] + ch, f01[q]);
+                        VecLoad<T, VEC>::ld(p10[q] + ch, f10[q]);
+                        VecLoad<T, VEC>::ld(p11[q] + ch, f11[q]);
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < UNR; ++q) {
+                    if (live[q]) {
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v)
+                            G[q] = __builtin_fmaf(g[q][v], bilerp(w00[q], w01[q], w10[q], w11[q], f00[q][v], f01[q][v], f10[q][v], f11[q][v]), G[q]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < UNR; ++q) {
+                float Gq = G[q];
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) {
+                    const float other = __shfl_down(Gq, off, kWave);
+                    if (lis + off < cp.lanes_per_slot) Gq += other;
+                }
+                if (live[q] && lis == 0) L.G[(it + q) * n_workers + worker] = Gq;
+            }
+        }
+    }
+
+    // ---- (4) rows, in groups of at most n_workers rows
+    for (int row_base = 0; row_base < k.H; row_base += n_workers) {
+        const int rows_here = min(n_workers, k.H - row_base);
+        for (int i = tid; i < rows_here; i += kColThreads) { L.rowcnt[i] = 0; L.rowfill[i] = 0; }
+        __syncthreads();
+        for (int e = tid; e < n_ent; e += kColThreads) {
+            const int vv = __float_as_int(L.entries[2 * e].y);
+            const int r0 = (vv & 0xffff) - row_base, r1 = ((vv >> 16) & 0xffff) - row_base;
+            if (r0 >= 0 && r0 < rows_here) atomicAdd(L.rowcnt + r0, 1);
+            if (r1 >= 0 && r1 < rows_here) atomicAdd(L.rowcnt + r1, 1);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            // prefix sum of the row lengths and slots per row: one each, the spare ones in proportion
+            int total = 0, nonempty = 0;
+            for (int r = 0; r < rows_here; ++r) { L.rowstart[r] = total; total += L.rowcnt[r]; nonempty += L.rowcnt[r] > 0; }
+            L.rowstart[rows_here] = total;
+            const int spare = n_workers - nonempty;
+            int w = 0;
+            for (int r = 0; r < rows_here; ++r) {
+                const int c = L.rowcnt[r];
+                if (c == 0) continue;
+                int n = 1 + (int)(((long long)spare * c) / total);
+                if (n > c) n = c;
+                for (int i = 0; i < n; ++i) { L.wk_row[w + i] = r; L.wk_first[w + i] = w; L.wk_n[w + i] = n; }
+                w += n;
+            }
+            for (; w < n_workers; ++w) L.wk_row[w] = -1;
+        }
+        __syncthreads();
+        for (int e = tid; e < n_ent; e += kColThreads) {
+            const int vv = __float_as_int(L.entries[2 * e].y);
+            const int r0 = (vv & 0xffff) - row_base, r1 = ((vv >> 16) & 0xffff) - row_base;
+            if (r0 >= 0 && r0 < rows_here) L.contrib[L.rowstart[r0] + atomicAdd(L.rowfill + r0, 1)] = e;
+            if (r1 >= 0 && r1 < rows_here) L.contrib[L.rowstart[r1] + atomicAdd(L.rowfill + r1, 1)] = e | (1 << 30);
+        }
+        __syncthreads();
+
+        // every slot gathers its share of one row into registers
+        const int my_row = carrier ? L.wk_row[worker] : -1;
+        float sa = 0.0f, sb = 0.0f;
+        for (int cb = 0; cb < k.C; cb += span) {
+            const int ch = cb + lis * VEC;
+            float acc[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+            if (my_row >= 0) {
+                const int part = worker - L.wk_first[worker], np = L.wk_n[worker];
+                const int lo = L.rowstart[my_row], hi = L.rowstart[my_row + 1];
+                constexpr int UNR = 1;
+                for (int j0 = lo + part; j0 < hi; j0 += np * UNR) {
+                    bool on[UNR];
+                    float coef[UNR], g[UNR][VEC];
+#pragma unroll
+                    for (int q = 0; q < UNR; ++q) {
+                        const int j = j0 + q * np;
+                        on[q] = j < hi;
+                        const int ce = L.contrib[on[q] ? j : lo];
+                        const int e = ce & 0x3fffffff;
+                        const bool second = (ce >> 30) & 1;             // this is the entry's v1 row
+                        const float4 e0 = L.entries[2 * e];
+                        const float4 e1 = L.entries[2 * e + 1];
+                        const int word = __float_as_int(e0.x);
+                        const bool c0 = (word >> 30) & 1, c1 = (word >> 31) & 1;
+                        const float du = e0.z, dv = e0.w;
+                        const float wv = second ? dv : 1.0f - dv;
+                        // my column's bilinear weight in this row, same products as the forward
+                        const float wc = (c0 ? (1.0f - du) * wv : 0.0f) + (c1 ? du * wv : 0.0f);
+                        coef[q] = e1.x * wc;
+                        if (on[q] && need_f && ch < k.C) {
+                            const float *go = grad_out + (size_t)(word & 0x3fffffff) * k.C + ch;
+                            VecLoad<float, VEC == 1 ? 1 : 4>::ld(go, *reinterpret_cast<float(*)[VEC == 1 ? 1 : 4]>(&g[q][0]));
+                            if (VEC == 8) VecLoad<float, 4>::ld(go + 4, *reinterpret_cast<float(*)[4]>(&g[q][VEC == 8 ? 4 : 0]));
+                        }
+                        if (on[q] && need_d && cb == 0 && lis == 0) {
+                            const float Gw = L.G[e] * wc;
+                            if (parametric) {
+                                sa = __builtin_fmaf(Gw, e1.y, sa);
+                                sb = __builtin_fmaf(Gw, e1.z, sb);
+                            } else {
+                                // two bins per contribution: the column is owned, the adds only meet
+                                // adds of this block
+                                const int kk = __float_as_int(e1.w);
+                                float *dst = d_depth + (size_t)((rowbase + row_base + my_row) * k.W + u) * Dd;
+                                atomic_add_f32(dst + (kk & 0xffff), Gw * e1.y);
+                                atomic_add_f32(dst + (kk >> 16), Gw * e1.z);
+                            }
+                        }
+                    }
+                    if (need_f && ch < k.C) {
+#pragma unroll
+                        for (int q = 0; q < UNR; ++q) {
+                            if (on[q]) {
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coef[q], g[q][v], acc[v]);
+                            }
+                        }
+                    }
+                }
+            }
+            if (cb > 0) __syncthreads();         // the previous channel block has been read
+            if (my_row >= 0) {
+                float *pw = L.part + (size_t)worker * cp.part_stride;
+                if (ch < k.C) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) pw[lis * VEC + v] = acc[v];
+                }
+                if (cb == 0 && lis == 0) { pw[span] = sa; pw[span + 1] = sb; }
+            }
+            __syncthreads();
+            // fixed-order sum of the partial rows; rows without contributions are written as
+            // zeros by the first flush so that the whole column is defined
+            const int width = min(span, k.C - cb);
+            for (int i = tid; i < rows_here * width; i += kColThreads) {
+                const int r = i / width, c = i - r * width;
+                float sum = 0.0f;
+                bool any = false;
+                for (int w = 0; w < n_workers; ++w) {
+                    if (L.wk_row[w] == r) { sum += L.part[(size_t)w * cp.part_stride + c]; any = true; }
+                }
+                if (need_f && (any || first_flush)) {
+                    float *dst = d_feats + (size_t)((rowbase + row_base + r) * k.W + u) * k.C + cb + c;
+                    *dst = (first_flush && !cp.accumulate) ? sum : *dst + sum;
+                }
+            }
+            if (cb == 0 && need_d && parametric) {
+                for (int i = tid; i < rows_here * 2; i += kColThreads) {
+                    const int r = i >> 1, c = i & 1;
+                    float sum = 0.0f;
+                    bool any = false;
+                    for (int w = 0; w < n_workers; ++w) {
+                        if (L.wk_row[w] == r) { sum += L.part[(size_t)w * cp.part_stride + span + c]; any = true; }
+                    }
+                    if (any || first_flush) {
+                        float *dst = d_depth + (size_t)((rowbase + row_base + r) * k.W + u) * 2 + c;
+                        *dst = (first_flush && !cp.accumulate) ? sum : *dst + sum;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kColThreads) void fbev_backward_column_kernel(
+    KParams k, ColParams cp, const float *__restrict__ grad_out, const T *__restrict__ depth,
+    const T *__restrict__ feats, const float *__restrict__ proj, const float *__restrict__ count,
+    float *__restrict__ d_depth, float *__restrict__ d_feats) {
+    extern __shared__ float4 smem[];
+    const int n_workers = kColWaves * cp.slots;
+    ColLds L;
+    L.Pm = reinterpret_cast<float *>(smem);
+    L.ctrl = reinterpret_cast<volatile int *>(smem + 4);
+    L.entries = smem + 8;
+    int *ip = reinterpret_cast<int *>(L.entries + 2 * kColEntries);
+    L.tiles = ip; ip += kColThreads;
+    L.cells = ip; ip += kColCells;
+    L.contrib = ip; ip += 2 * kColEntries;
+    L.rowcnt = ip; ip += kColMaxRows;
+    L.rowstart = ip; ip += kColMaxRows + 4;
+    L.rowfill = ip; ip += kColMaxRows;
+    L.wk_row = ip; ip += 64;
+    L.wk_first = ip; ip += 64;
+    L.wk_n = ip; ip += 64;
+    L.G = reinterpret_cast<float *>(ip); ip += kColEntries;
+    L.part = reinterpret_cast<float *>(ip);
+    (void)n_workers;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int bid = xcd_swizzle(blockIdx.x, cp.n_blocks);
+    const int u = bid % k.W;
+    const int cam = (bid / k.W) % k.N;
+    const int b = bid / (k.W * k.N);
+    const int Dd = k.Dd;
+    const int rowbase = (b * k.N + cam) * k.H;
+
+    if (tid < 12) L.Pm[tid] = proj[(size_t)(b * k.N + cam) * k.proj_stride + tid];
+    if (tid < 4) L.ctrl[tid] = 0;
+    // the categorical depth gradient is added with atomics below: define the owned region first
+    if (d_depth != nullptr && k.dist == FBEV_CATEGORICAL && !cp.accumulate) {
+        for (int i = tid; i < k.H * Dd; i += kColThreads)
+            d_depth[(size_t)((rowbase + i / Dd) * k.W + u) * Dd + (i % Dd)] = 0.0f;
+        __threadfence();
+    }
+    __syncthreads();
+    const float *Pm = L.Pm;
+
+    const float z_lo = voxel_coord(k.zmin, 0, k.vz), z_hi = voxel_coord(k.zmin, k.gz - 1, k.vz);
+    const float u_lo = (float)(u - 1) - kCullMargin, u_hi = (float)(u + 1) + kCullMargin;
+    bool first_flush = true;
+
+    for (int tile_base = 0; tile_base < cp.n_tiles; tile_base += kColThreads) {
+        // ---- (1a) tiles: one per thread
+        {
+            const int tile = tile_base + tid;
+            bool keep = false;
+            if (tile < cp.n_tiles) {
+                const int ty = tile / k.tiles_x, tx = tile - ty * k.tiles_x;
+                const int ix0 = tx * kTile, ix1 = min(ix0 + kTile, k.gx) - 1;
+                const int iy0 = ty * kTile, iy1 = min(iy0 + kTile, k.gy) - 1;
+                const float xs[2] = {voxel_coord(k.xmin, ix0, k.vx), voxel_coord(k.xmin, ix1, k.vx)};
+                const float ys[2] = {voxel_coord(k.ymin, iy0, k.vy), voxel_coord(k.ymin, iy1, k.vy)};
+                const float zs[2] = {z_lo, z_hi};
+                float fu_min = 3.0e38f, fu_max = -3.0e38f, fv_min = 3.0e38f, fv_max = -3.0e38f, d_min = 3.0e38f,
+                      d_max = -3.0e38f;
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const float x = xs[c & 1], y = ys[(c >> 1) & 1], z = zs[c >> 2];
+                    const float U = ((Pm[0] * x + Pm[1] * y) + Pm[2] * z) + Pm[3];
+                    const float V = ((Pm[4] * x + Pm[5] * y) + Pm[6] * z) + Pm[7];
+                    const float D = ((Pm[8] * x + Pm[9] * y) + Pm[10] * z) + Pm[11];
+                    d_min = fminf(d_min, D);
+                    d_max = fmaxf(d_max, D);
+                    const float dc = fmaxf(D, kCullNear);
+                    const float fu = ((U / dc) / k.Wi_f) * k.W_f, fv = ((V / dc) / k.Hi_f) * k.H_f;
+                    fu_min = fminf(fu_min, fu); fu_max = fmaxf(fu_max, fu);
+                    fv_min = fminf(fv_min, fv); fv_max = fmaxf(fv_max, fv);
+                }
+                if (!(d_max > -1.0e-3f)) keep = false;                 // the whole box is behind the camera
+                else if (!(d_min > kCullNear)) keep = true;            // too close to the camera plane to bound u
+                else keep = fu_max >= u_lo && fu_min < u_hi && fv_max >= -kCullMargin &&
+                            fv_min < k.H_f + kCullMargin;
+            }
+            const int pos = wave_append(&L.ctrl[0], keep, lane);
+            if (keep) L.tiles[pos] = tile_base + tid;
+        }
+        __syncthreads();
+        const int n_tiles_kept = L.ctrl[0];
+
+        for (int tb = 0; tb < n_tiles_kept; tb += kColCells / 64) {
+            // ---- (1b) cells of up to 32 kept tiles: u-range over the cell's height segment
+            const int n_cell_tests = min(kColCells / 64, n_tiles_kept - tb) * 64;
+            for (int c0 = 0; c0 < n_cell_tests; c0 += kColThreads) {
+                const int ci = c0 + tid;
+                bool keep = false;
+                int packed = 0;
+                if (ci < n_cell_tests) {
+                    const int tile = L.tiles[tb + (ci >> 6)];
+                    const int ty = tile / k.tiles_x, tx = tile - ty * k.tiles_x;
+                    const int ix = tx * kTile + (ci & 7), iy = ty * kTile + ((ci >> 3) & 7);
+                    if (ix < k.gx && iy < k.gy) {
+                        const float x = voxel_coord(k.xmin, ix, k.vx), y = voxel_coord(k.ymin, iy, k.vy);
+                        const float Uxy = Pm[0] * x + Pm[1] * y, Dxy = Pm[8] * x + Pm[9] * y;
+                        const float Ua = (Uxy + Pm[2] * z_lo) + Pm[3], Da = (Dxy + Pm[10] * z_lo) + Pm[11];
+                        const float Ub = (Uxy + Pm[2] * z_hi) + Pm[3], Db = (Dxy + Pm[10] * z_hi) + Pm[11];
+                        const float dmin = fminf(Da, Db), dmax = fmaxf(Da, Db);
+                        if (!(dmax > -1.0e-3f)) keep = false;
+                        else if (!(dmin > kCullNear)) keep = true;
+                        else {
+                            const float fa = ((Ua / Da) / k.Wi_f) * k.W_f, fb = ((Ub / Db) / k.Wi_f) * k.W_f;
+                            keep = fmaxf(fa, fb) >= u_lo && fminf(fa, fb) < u_hi;
+                        }
+                        packed = ix | (iy << 16);
+                    }
+                }
+                const int pos = wave_append(&L.ctrl[1], keep, lane);
+                if (keep) L.cells[pos] = packed;
+            }
+            __syncthreads();
+            const int n_cells = L.ctrl[1];
+            const int n_samples = n_cells * k.gz;
+
+            // ---- (2) samples of the kept cells, one per thread and round
+            for (int s0 = 0; s0 < n_samples; s0 += kColThreads) {
+                {
+                    const int idx = s0 + tid;
+                    bool keep = false;
+                    float4 e0 = make_float4(0.f, 0.f, 0.f, 0.f), e1 = e0;
+                    if (idx < n_samples) {
+                        const int ci = idx / k.gz, iz = idx - ci * k.gz;
+                        const int packed = L.cells[ci];
+                        const int ix = packed & 0xffff, iy = packed >> 16;
+                        Geom g = project_sample(k, Pm, voxel_coord(k.xmin, ix, k.vx), voxel_coord(k.ymin, iy, k.vy),
+                                                voxel_coord(k.zmin, iz, k.vz));
+                        const bool c0 = g.u0 == u, c1 = g.u1 == u;
+                        if (g.valid && (c0 || c1)) {
+                            const float w00 = (1.0f - g.du) * (1.0f - g.dv), w01 = (1.0f - g.du) * g.dv;
+                            const float w10 = g.du * (1.0f - g.dv), w11 = g.du * g.dv;
+                            const int t00 = (rowbase + g.v0) * k.W + g.u0, t01 = (rowbase + g.v1) * k.W + g.u0;
+                            const int t10 = (rowbase + g.v0) * k.W + g.u1, t11 = (rowbase + g.v1) * k.W + g.u1;
+                            DepthEval e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
+                            if (e.keep) {
+                                const int cell = (b * k.gy + iy) * k.gx + ix;
+                                const float n = count[cell];
+                                const float inv = k.reduce_sum ? 1.0f : (n > 0.0f ? 1.0f / n : 0.0f);
+                                keep = true;
+                                e0 = make_float4(__int_as_float(cell | (c0 ? (1 << 30) : 0) | (c1 ? (1 << 31) : 0)),
+                                                 __int_as_float(g.v0 | (g.v1 << 16)), g.du, g.dv);
+                                e1 = make_float4(e.wgt * inv, e.a * inv, e.b * inv, __int_as_float(e.k0 | (e.k1 << 16)));
+                            }
+                        }
+                    }
+                    const int pos = wave_append(&L.ctrl[2], keep, lane);
+                    if (keep) {
+                        L.entries[2 * pos] = e0;
+                        L.entries[2 * pos + 1] = e1;
+                    }
+                }
+                __syncthreads();
+                const int n_ent = L.ctrl[2];
+                if (n_ent + kColThreads > kColEntries) {
+                    column_consume<T, VEC>(k, cp, L, n_ent, u, rowbase, first_flush, grad_out, feats, d_depth, d_feats);
+                    first_flush = false;
+                    __syncthreads();
+                    if (tid == 0) L.ctrl[2] = 0;
+                    __syncthreads();
+                }
+            }
+            __syncthreads();
+            if (tid == 0) L.ctrl[1] = 0;
+            __syncthreads();
+        }
+        __syncthreads();
+        if (tid == 0) L.ctrl[0] = 0;
+        __syncthreads();
+    }
+    // whatever is left, and in any case one flush so that every element of the column is written
+    const int n_ent = L.ctrl[2];
+    if (n_ent > 0 || first_flush)
+        column_consume<T, VEC>(k, cp, L, n_ent, u, rowbase, first_flush, grad_out, feats, d_depth, d_feats);
 }
 
 // ---------------------------------------------------------------- geometry inspection
@@ -952,16 +1439,49 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan) {
 
 template <typename T, int VEC>
 int launch_forward(const Plan &pl, const void *depth, const void *feats, const float *proj, float *out,
-                   hipStream_t st) {
+                   float *cnt, hipStream_t st) {
     dim3 grid(pl.k.n_blocks), block(kWave * kWavesPerBlock);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
-    prof::Scope timer(prof::kForward, st);
+    prof::Scope timer(out != nullptr ? prof::kForward : prof::kCellCount, st);
     switch (pl.cpl) {
-        case 1: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 1>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out); break;
-        case 2: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 2>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out); break;
-        default: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 4>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out); break;
+        case 1: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 1>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
+        case 2: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 2>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
+        default: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 4>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
     }
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+int dispatch_forward(const fbev_problem *p, const Plan &pl, const void *depth, const void *feats, const float *proj,
+                     float *out, float *cnt, hipStream_t st) {
+    switch (p->in_dtype) {
+        case FBEV_F32:
+            return pl.vec == 4 ? launch_forward<float, 4>(pl, depth, feats, proj, out, cnt, st)
+                               : launch_forward<float, 1>(pl, depth, feats, proj, out, cnt, st);
+        case FBEV_F16:
+            return pl.vec == 8 ? launch_forward<__half, 8>(pl, depth, feats, proj, out, cnt, st)
+                               : launch_forward<__half, 1>(pl, depth, feats, proj, out, cnt, st);
+        default:
+            return pl.vec == 8 ? launch_forward<bf16_raw, 8>(pl, depth, feats, proj, out, cnt, st)
+                               : launch_forward<bf16_raw, 1>(pl, depth, feats, proj, out, cnt, st);
+    }
+}
+
+template <typename T, int VEC>
+int launch_columns(const Plan &pl, const ColParams &cp, size_t lds, const float *go, const void *depth,
+                   const void *feats, const float *proj, const float *count, float *dd, float *df, hipStream_t st) {
+    auto kernel = fbev_backward_column_kernel<T, VEC>;
+    // more than 64 KiB of dynamic LDS has to be opted into, once per kernel and size
+    static std::atomic<size_t> opted_in{(size_t)kMaxBlockLdsBytes};
+    if (lds > opted_in.load(std::memory_order_relaxed)) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess)
+            return FBEV_ERR_LAUNCH;
+        opted_in.store(lds, std::memory_order_relaxed);
+    }
+    prof::Scope timer(prof::kBackwardColumn, st);
+    hipLaunchKernelGGL(kernel, dim3(cp.n_blocks), dim3(kColThreads), lds, st, pl.k, cp, go,
+                       static_cast<const T *>(depth), static_cast<const T *>(feats), proj, count, dd, df);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
@@ -1024,6 +1544,18 @@ size_t ws_index_bytes(const fbev_problem *p) {
     return ((size_t)(counter_count(p) + chunk_count(p) + 1) * sizeof(int) + 255) / 256 * 256;
 }
 
+int launch_zero(int *a, long long na, float *b, long long nb, float *c, long long nc, hipStream_t st) {
+    if (!a) na = 0;
+    if (!b) nb = 0;
+    if (!c) nc = 0;
+    const long long n = na + nb + nc;
+    if (n == 0) return FBEV_OK;
+    prof::Scope timer(prof::kZero, st);
+    hipLaunchKernelGGL(fbev_fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a, na,
+                       reinterpret_cast<int *>(b), nb, reinterpret_cast<int *>(c), nc);
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
 int check_backward_args(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
                         const float *proj, const float *d_depth, const float *d_feats) {
     if (!grad_out || !depth || !feats || !proj) return FBEV_ERR_NULL;
@@ -1039,33 +1571,23 @@ int check_backward_args(const fbev_problem *p, const float *grad_out, const void
 extern "C" {
 
 int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, const float *proj, float *out,
-                 void *stream) {
+                 float *count_out, void *stream) {
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
     if (!depth || !feats || !proj || !out) return FBEV_ERR_NULL;
     const int es = elem_size(p->in_dtype);
-    if ((uintptr_t)depth % es || (uintptr_t)feats % es || (uintptr_t)proj % 4 || (uintptr_t)out % 4)
+    if ((uintptr_t)depth % es || (uintptr_t)feats % es || (uintptr_t)proj % 4 || (uintptr_t)out % 4 ||
+        (uintptr_t)count_out % 4)
         return FBEV_ERR_ALIGNMENT;
     Plan pl;
     // 128-bit gathers and stores need 16-byte aligned feature and result tensors
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl);
     if (rc != FBEV_OK) return rc;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (p->in_dtype) {
-        case FBEV_F32:
-            return pl.vec == 4 ? launch_forward<float, 4>(pl, depth, feats, proj, out, st)
-                               : launch_forward<float, 1>(pl, depth, feats, proj, out, st);
-        case FBEV_F16:
-            return pl.vec == 8 ? launch_forward<__half, 8>(pl, depth, feats, proj, out, st)
-                               : launch_forward<__half, 1>(pl, depth, feats, proj, out, st);
-        default:
-            return pl.vec == 8 ? launch_forward<bf16_raw, 8>(pl, depth, feats, proj, out, st)
-                               : launch_forward<bf16_raw, 1>(pl, depth, feats, proj, out, st);
-    }
+    return dispatch_forward(p, pl, depth, feats, proj, out, count_out, static_cast<hipStream_t>(stream));
 }
 
 int fbev_backward(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
-                  const float *proj, float *d_depth, float *d_feats, void *stream) {
+                  const float *proj, float *d_depth, float *d_feats, int accumulate, void *stream) {
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
     rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
@@ -1074,8 +1596,67 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
     Plan pl;
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl);
     if (rc != FBEV_OK) return rc;
+    if (!accumulate) {
+        rc = launch_zero(nullptr, 0, d_depth, texel_count(p) * p->depth_bins, d_feats, texel_count(p) * p->channels,
+                         static_cast<hipStream_t>(stream));
+        if (rc != FBEV_OK) return rc;
+    }
     return dispatch_cells<false>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, nullptr, nullptr, nullptr, 0,
                                  static_cast<hipStream_t>(stream));
+}
+
+size_t fbev_backward_columns_workspace_bytes(const fbev_problem *p) {
+    if (validate(p, true) != FBEV_OK) return 0;
+    return ((size_t)p->batch * p->grid_y * p->grid_x * sizeof(float) + 255) / 256 * 256;
+}
+
+int fbev_backward_columns(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                          const float *proj, const float *cell_count, float *d_depth, float *d_feats,
+                          int accumulate, void *workspace, size_t workspace_bytes, void *stream) {
+    int rc = validate(p, true);
+    if (rc != FBEV_OK) return rc;
+    rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
+    if (rc != FBEV_OK) return rc;
+    if ((uintptr_t)cell_count % 4 || (uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
+    if (!d_depth && !d_feats) return FBEV_OK;
+    if (p->feat_h > 0xffff || (long long)p->batch * p->grid_y * p->grid_x >= (1ll << 30)) return FBEV_ERR_TOO_LARGE;
+    Plan pl;
+    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl);
+    if (rc != FBEV_OK) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (cell_count == nullptr) {
+        // recount: the forward's sample phase alone, counts into the workspace
+        if (!workspace) return FBEV_ERR_NULL;
+        if (workspace_bytes < fbev_backward_columns_workspace_bytes(p)) return FBEV_ERR_SHAPE;
+        rc = dispatch_forward(p, pl, depth, feats, proj, nullptr, static_cast<float *>(workspace), st);
+        if (rc != FBEV_OK) return rc;
+        cell_count = static_cast<const float *>(workspace);
+    }
+    ColParams cp;
+    cp.n_tiles = pl.k.tiles_x * pl.k.tiles_y;
+    const int cq = (p->channels + pl.vec - 1) / pl.vec;
+    cp.lanes_per_slot = cq < kWave ? cq : kWave;
+    cp.slots = kWave / cp.lanes_per_slot;
+    if (cp.slots * kColWaves > 64) cp.slots = 64 / kColWaves;
+    cp.part_stride = (cp.lanes_per_slot * pl.vec + 2 + 3) / 4 * 4;
+    cp.accumulate = accumulate != 0;
+    cp.n_blocks = p->batch * p->num_cams * p->feat_w;
+    if (p->feat_h > kColMaxRows || p->grid_x > 0xffff || p->grid_y > 0x7fff) return FBEV_ERR_TOO_LARGE;
+    const size_t ints = (size_t)kColThreads + kColCells + 2 * kColEntries + 3 * kColMaxRows + 4 + 3 * 64 + kColEntries;
+    const size_t lds = 8 * sizeof(float4) + (size_t)kColEntries * 32 + ints * sizeof(int) +
+                       (size_t)kColWaves * cp.slots * cp.part_stride * sizeof(float);
+    if (lds > 150 * 1024) return FBEV_ERR_TOO_LARGE;
+    switch (p->in_dtype) {
+        case FBEV_F32:
+            return pl.vec == 4 ? launch_columns<float, 4>(pl, cp, lds, grad_out, depth, feats, proj, cell_count, d_depth, d_feats, st)
+                               : launch_columns<float, 1>(pl, cp, lds, grad_out, depth, feats, proj, cell_count, d_depth, d_feats, st);
+        case FBEV_F16:
+            return pl.vec == 8 ? launch_columns<__half, 8>(pl, cp, lds, grad_out, depth, feats, proj, cell_count, d_depth, d_feats, st)
+                               : launch_columns<__half, 1>(pl, cp, lds, grad_out, depth, feats, proj, cell_count, d_depth, d_feats, st);
+        default:
+            return pl.vec == 8 ? launch_columns<bf16_raw, 8>(pl, cp, lds, grad_out, depth, feats, proj, cell_count, d_depth, d_feats, st)
+                               : launch_columns<bf16_raw, 1>(pl, cp, lds, grad_out, depth, feats, proj, cell_count, d_depth, d_feats, st);
+    }
 }
 
 uint64_t fbev_backward_max_pairs(const fbev_problem *p) {
@@ -1089,7 +1670,7 @@ size_t fbev_backward_workspace_bytes(const fbev_problem *p, uint64_t pair_capaci
 }
 
 int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
-                         const float *proj, float *d_depth, float *d_feats, void *workspace,
+                         const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
                          size_t workspace_bytes, void *stream) {
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
@@ -1114,12 +1695,9 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const long long counters = counter_count(p), chunks = chunk_count(p);
     int *chunk_prefix = cursor + counters;
 
-    {
-        prof::Scope timer(prof::kZero, st);
-        hipLaunchKernelGGL(fbev_fill_zero_kernel, dim3((unsigned)((counters + 255) / 256)), dim3(256), 0, st, cursor,
-                           counters);
-    }
-    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+    rc = launch_zero(cursor, counters, accumulate ? nullptr : d_depth, texels * p->depth_bins,
+                     accumulate ? nullptr : d_feats, texels * p->channels, st);
+    if (rc != FBEV_OK) return rc;
     switch (p->in_dtype) {
         case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, samples, st); break;
         case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, samples, st); break;
@@ -1151,10 +1729,10 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const int from_pairs = (d_depth != nullptr && p->depth_distribution != FBEV_CATEGORICAL) ? 1 : 0;
     prof::Scope timer(prof::kBackwardTexel, st);
     if (vec4)
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels), dim3(kWave * kWavesPerBlock), lds,
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels, kTexelSplit), dim3(kWave * kWavesPerBlock), lds,
                            st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
     else
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels), dim3(kWave * kWavesPerBlock), lds,
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels, kTexelSplit), dim3(kWave * kWavesPerBlock), lds,
                            st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }

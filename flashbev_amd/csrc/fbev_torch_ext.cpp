@@ -143,7 +143,7 @@ void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &ima
                            float voxel_z_min, at::Tensor out, int64_t total_threads, int depth_distribution,
                            bool use_shared_memory, bool optimize_z_precompute, bool use_warp_kernel,
                            bool use_vectorized_load, float epsilon, float depth_weight_threshold,
-                           float depth_min, float depth_step, int reduction) {
+                           float depth_min, float depth_step, int reduction, std::optional<at::Tensor> count_out) {
     (void)use_shared_memory; (void)optimize_z_precompute; (void)use_warp_kernel; (void)use_vectorized_load;
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
@@ -157,10 +157,17 @@ void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &ima
                 p.channels, "], got ", out.sizes());
     TORCH_CHECK(total_threads == out.numel(), "flashbevpool_ext: total_threads (", total_threads,
                 ") must equal out.numel() (", out.numel(), ")");
+    float *cnt = nullptr;
+    if (count_out.has_value() && count_out->defined()) {
+        check_dev(*count_out, depth_params, "count_out");
+        TORCH_CHECK(count_out->scalar_type() == at::kFloat && count_out->numel() == (int64_t)p.batch * p.grid_y * p.grid_x,
+                    "flashbevpool_ext: count_out must be float32 [B,grid_y,grid_x]");
+        cnt = count_out->data_ptr<float>();
+    }
     DeviceScope scope(depth_params.get_device());
     hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
     raise_on(fbev_forward(&p, depth_params.data_ptr(), image_feats.data_ptr(), projection_matrices.data_ptr<float>(),
-                          out.data_ptr<float>(), st),
+                          out.data_ptr<float>(), cnt, st),
              "fbev_forward");
 }
 
@@ -173,7 +180,7 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                             std::optional<at::Tensor> depth_params_grad, std::optional<at::Tensor> image_feats_grad,
                             int64_t total_threads, int depth_distribution, float epsilon, float depth_weight_threshold,
                             float depth_min, float depth_step, int reduction, int backward_mode,
-                            int64_t pair_capacity) {
+                            int64_t pair_capacity, std::optional<at::Tensor> cell_count, bool accumulate) {
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
     auto roi = host_floats(roi_range, 6, "roi_range");
@@ -205,25 +212,54 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
     }
     DeviceScope scope(depth_params.get_device());
     hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
-    TORCH_CHECK(backward_mode >= 0 && backward_mode <= 2,
-                "flashbevpool_ext: backward_mode must be 0 (auto), 1 (atomic scatter) or 2 (inverse-map gather)");
-    if (backward_mode == 1) {
-        raise_on(fbev_backward(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
-                               projection_matrices.data_ptr<float>(), dd, df, st),
-                 "fbev_backward");
-        return;
-    }
+    TORCH_CHECK(backward_mode >= 0 && backward_mode <= 3,
+                "flashbevpool_ext: backward_mode must be 0 (auto), 1 (atomic scatter), 2 (inverse-map gather) or "
+                "3 (column owner)");
+    auto run_columns = [&]() -> int {
+        const float *cnt = nullptr;
+        at::Tensor ws;
+        size_t ws_bytes = 0;
+        if (cell_count.has_value() && cell_count->defined()) {
+            check_dev(*cell_count, depth_params, "cell_count");
+            TORCH_CHECK(cell_count->scalar_type() == at::kFloat &&
+                            cell_count->numel() == (int64_t)p.batch * p.grid_y * p.grid_x,
+                        "flashbevpool_ext: cell_count must be float32 [B,grid_y,grid_x]");
+            cnt = cell_count->data_ptr<float>();
+        } else {
+            ws_bytes = fbev_backward_columns_workspace_bytes(&p);
+            ws = at::empty({(int64_t)ws_bytes}, at::TensorOptions().device(depth_params.device()).dtype(at::kByte));
+        }
+        return fbev_backward_columns(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                                     projection_matrices.data_ptr<float>(), cnt, dd, df, accumulate ? 1 : 0,
+                                     ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, st);
+    };
     // Inverse-map gather.  The pair array comes from PyTorch's caching allocator (no device
     // allocation in steady state).  Half of the worst case holds every rig whose cameras see
     // less than half of all (cell, height) samples; what does not fit is applied with atomics.
-    const uint64_t max_pairs = fbev_backward_max_pairs(&p);
-    uint64_t cap = pair_capacity >= 0 ? (uint64_t)pair_capacity : (max_pairs + 1) / 2;
-    if (cap > max_pairs) cap = max_pairs;
-    const size_t bytes = fbev_backward_workspace_bytes(&p, cap);
-    at::Tensor ws = at::empty({(int64_t)bytes}, at::TensorOptions().device(depth_params.device()).dtype(at::kByte));
-    raise_on(fbev_backward_gather(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
-                                  projection_matrices.data_ptr<float>(), dd, df, ws.data_ptr(), bytes, st),
-             "fbev_backward_gather");
+    auto run_gather = [&]() -> int {
+        const uint64_t max_pairs = fbev_backward_max_pairs(&p);
+        uint64_t cap = pair_capacity >= 0 ? (uint64_t)pair_capacity : (max_pairs + 1) / 2;
+        if (cap > max_pairs) cap = max_pairs;
+        const size_t bytes = fbev_backward_workspace_bytes(&p, cap);
+        at::Tensor ws = at::empty({(int64_t)bytes}, at::TensorOptions().device(depth_params.device()).dtype(at::kByte));
+        return fbev_backward_gather(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                                    projection_matrices.data_ptr<float>(), dd, df, accumulate ? 1 : 0, ws.data_ptr(),
+                                    bytes, st);
+    };
+    if (backward_mode == 1) {
+        raise_on(fbev_backward(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                               projection_matrices.data_ptr<float>(), dd, df, accumulate ? 1 : 0, st),
+                 "fbev_backward");
+    } else if (backward_mode == 2) {
+        raise_on(run_gather(), "fbev_backward_gather");
+    } else if (backward_mode == 3) {
+        raise_on(run_columns(), "fbev_backward_columns");
+    } else {
+        // auto: the inverse map; problems beyond its 32-bit pair positions go to the column owner
+        int rc = run_gather();
+        if (rc == FBEV_ERR_TOO_LARGE) raise_on(run_columns(), "fbev_backward_columns");
+        else raise_on(rc, "fbev_backward_gather");
+    }
 }
 
 // Parity hook: per-sample validity mask and bilinear corner indices, [B,gy,gx,N,gz(,4|2)].
@@ -272,14 +308,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("out"), py::arg("total_threads"), py::arg("depth_distribution"), py::arg("use_shared_memory"),
           py::arg("optimize_z_precompute"), py::arg("use_warp_kernel"), py::arg("use_vectorized_load"),
           py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f, py::arg("depth_min") = 1.0f,
-          py::arg("depth_step") = 1.0f, py::arg("reduction") = 0);
+          py::arg("depth_step") = 1.0f, py::arg("reduction") = 0, py::arg("count_out") = py::none());
     m.def("flash_bevpool_backward", &flash_bevpool_backward, "fused camera->BEV pooling, backward",
           py::arg("out_grad"), py::arg("depth_params"), py::arg("image_feats"), py::arg("projection_matrices"),
           py::arg("feature_size"), py::arg("image_size"), py::arg("roi_range"), py::arg("grid_size"),
           py::arg("depth_params_grad"), py::arg("image_feats_grad"), py::arg("total_threads"),
           py::arg("depth_distribution"), py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f,
           py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0,
-          py::arg("backward_mode") = 0, py::arg("pair_capacity") = -1);
+          py::arg("backward_mode") = 0, py::arg("pair_capacity") = -1, py::arg("cell_count") = py::none(),
+          py::arg("accumulate") = true);
     m.def("sample_geometry", &sample_geometry, "per-sample validity mask and corner indices (parity hook)",
           py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
           py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);

@@ -33,9 +33,10 @@ import torch
 from ._native import load_ext
 
 _SUPPORTED = (torch.float32, torch.float16, torch.bfloat16)
-# how the backward pass forms the feature gradient: "gather" (inverse map, no float atomics,
-# the default) or "scatter" (hardware fp32 atomics, no workspace)
-_BACKWARD_MODES = {"auto": 0, "scatter": 1, "gather": 2}
+# how the backward pass forms the gradients: "gather" (texel inverse map; what "auto" picks),
+# "columns" (one workgroup owns a feature-map column: no workspace, no global atomics on the
+# feature gradient) or "scatter" (fp32 atomics, no workspace)
+_BACKWARD_MODES = {"auto": 0, "scatter": 1, "gather": 2, "columns": 3}
 
 
 def _backward_mode() -> int:
@@ -126,14 +127,19 @@ class FlashBEVPool(torch.autograd.Function):
 
         out = torch.empty((B, grid[1], grid[0], C), dtype=torch.float32, device=image_feats.device)
         red = 0 if reduction == "mean" else 1
+        # the per-cell sample counts cost the forward nothing and save the backward a recount
+        wants_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        counts = torch.empty((B, grid[1], grid[0]), dtype=torch.float32,
+                             device=image_feats.device) if wants_grad else None
         ext.flash_bevpool_forward(
             depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
             vsize[0], vsize[1], vsize[2], vmin[0], vmin[1], vmin[2], out, out.numel(),
             depth_distribution, bool(use_shared_memory), bool(optimize_z_precompute),
             bool(use_warp_kernel), bool(use_vectorized_load), float(epsilon),
-            float(depth_weight_threshold), d_min, d_step, red)
+            float(depth_weight_threshold), d_min, d_step, red, counts)
 
         ctx.save_for_backward(depth_params, image_feats, projection_matrices)
+        ctx.counts = counts
         ctx.host = (fs_host, image_t, roi_t, grid_t)
         ctx.total_threads = out.numel()
         ctx.depth_distribution = depth_distribution
@@ -149,16 +155,20 @@ class FlashBEVPool(torch.autograd.Function):
         depth_params, image_feats, projection_matrices = ctx.saved_tensors
         fs_host, image_t, roi_t, grid_t = ctx.host
         need_depth, need_feats = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        depth_params_grad = torch.zeros(depth_params.shape, dtype=torch.float32,
-                                        device=depth_params.device) if need_depth else None
-        image_feats_grad = torch.zeros(image_feats.shape, dtype=torch.float32,
-                                       device=image_feats.device) if need_feats else None
+        mode = _backward_mode()
+        # the library defines every gradient element itself (accumulate = False), so the buffers
+        # need no zero-fill of their own (the reference fills them, flash_bevpool.py:115-116)
+        alloc = torch.empty
+        depth_params_grad = alloc(depth_params.shape, dtype=torch.float32,
+                                  device=depth_params.device) if need_depth else None
+        image_feats_grad = alloc(image_feats.shape, dtype=torch.float32,
+                                 device=image_feats.device) if need_feats else None
         if need_depth or need_feats:
             ext.flash_bevpool_backward(
                 out_grad.contiguous().float(), depth_params, image_feats, projection_matrices,
                 fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
                 ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
-                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, _backward_mode(), -1)
+                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, -1, ctx.counts, False)
         return (depth_params_grad, image_feats_grad) + (None,) * 14
 
 

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 1
+#define FBEV_ABI_VERSION 2
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -75,32 +75,36 @@ typedef struct fbev_problem {
 /*
  * Forward: out[b,y,x,:] = mean (or sum) over the valid (camera, height-bin) samples of
  * depth_weight * bilinear(feats).  Every element of `out` is written (cells that no
- * camera sees get 0), so `out` need not be zeroed.
+ * camera sees get 0), so `out` need not be zeroed.  If `count_out` is not NULL it receives,
+ * as float [B, grid_y, grid_x], the number of samples that entered each cell's mean (what the
+ * reference keeps in `valid_count`, flash_bevpool_cuda.cu:198-216); fbev_backward_columns can
+ * reuse it.
  * Replaces the launcher flash_bevpool(...) (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:757-865)
  * as bound by flash_bevpool_forward (flashbev/flashbevpool/src/flash_bevpool.cpp:79-166).
  */
 int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, const float *proj,
-                 float *out, void *stream);
+                 float *out, float *count_out, void *stream);
 
 /*
- * Backward: ACCUMULATES the exact gradients of fbev_forward into d_depth and d_feats, which
- * the caller zero-fills (the reference's ownership rule, flashbev/flashbevpool/flash_bevpool.py:115-116).
- * Either gradient pointer may be NULL to skip that gradient.
+ * Backward: the exact gradients of fbev_forward.  With accumulate != 0 they are ADDED to
+ * d_depth and d_feats, which the caller has zero-filled (the reference's ownership rule,
+ * flashbev/flashbevpool/flash_bevpool.py:115-116); with accumulate == 0 the library defines
+ * every element itself (the zero-fill is folded into its first launch) and the buffers may
+ * hold anything.  Either gradient pointer may be NULL to skip that gradient.
  * Replaces flash_bevpool_grad(...) (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:867-937) as bound by
  * flash_bevpool_backward (flashbev/flashbevpool/src/flash_bevpool.cpp:168-241).  The depth gradient is
  * the true derivative of the forward, not the reference kernel's expression at
  * flash_bevpool_cuda.cu:665-674.
  */
 int fbev_backward(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
-                  const float *proj, float *d_depth, float *d_feats, void *stream);
+                  const float *proj, float *d_depth, float *d_feats, int accumulate, void *stream);
 
 /*
  * Backward through an inverse map (texel -> contributing samples): the same gradients as
  * fbev_backward, formed without floating-point atomics on the feature gradient.  The call
  * counts the contributing sample corners per texel, prefix-sums the counts, writes one
  * 16-byte (cell, coefficient) pair per corner into the texel's segment of the workspace and
- * then gathers per texel.  It ACCUMULATES into the zero-filled d_depth / d_feats like
- * fbev_backward.  `workspace` is caller-owned device memory, 16-byte aligned, of at least
+ * then gathers per texel.  `accumulate` as in fbev_backward.  `workspace` is caller-owned device memory, 16-byte aligned, of at least
  * fbev_backward_workspace_bytes(p, 0) bytes; pairs that do not fit its capacity are applied
  * with atomics instead, so any capacity gives correct results and
  * fbev_backward_workspace_bytes(p, fbev_backward_max_pairs(p)) never overflows.  The
@@ -111,8 +115,29 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
  * applied to the forward pass.
  */
 int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
-                         const float *proj, float *d_depth, float *d_feats, void *workspace,
+                         const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
                          size_t workspace_bytes, void *stream);
+
+/*
+ * Backward by column ownership: the same gradients again, one launch, no global atomics and
+ * no pair lists.  One workgroup owns one feature-map column (b, camera, u), finds the BEV
+ * tiles whose samples can reach it, re-projects those samples, gathers the grad_out rows and
+ * accumulates the column's gradient in LDS, then stores it.  Every element of d_depth and
+ * d_feats is written by exactly one workgroup: with accumulate = 0 the buffers need not be
+ * zero-filled (they are overwritten), with accumulate != 0 the result is added to them as in
+ * fbev_backward.  `cell_count` is the count_out of fbev_forward for the same inputs; if it is
+ * NULL the counts are recomputed into `workspace` (at least
+ * fbev_backward_columns_workspace_bytes(p) bytes, 16-byte aligned), which is otherwise unused
+ * and may be NULL.  Limits: feat_h * (channels + depth_bins) * 4 bytes must fit LDS beside the
+ * sample buffer (about 80 KiB), feat_h <= 65535.
+ * Replaces flash_bevpool_grad(...) (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:867-937) like
+ * fbev_backward does.
+ */
+int fbev_backward_columns(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                          const float *proj, const float *cell_count, float *d_depth, float *d_feats,
+                          int accumulate, void *workspace, size_t workspace_bytes, void *stream);
+
+size_t fbev_backward_columns_workspace_bytes(const fbev_problem *p);
 
 /* Upper bound of the pairs one backward call can produce: 4 corners per (cell, camera, height) sample. */
 uint64_t fbev_backward_max_pairs(const fbev_problem *p);

@@ -61,40 +61,59 @@ def problem_for(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN)
                              reduction=reduction, proj_stride=x["projection_matrices"].shape[-2] * 4)
 
 
-def capi_forward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN):
-    """Forward through the C ABI on the tensors' device; returns out [B,gy,gx,C] float32."""
+def capi_forward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, with_count=False):
+    """Forward through the C ABI on the tensors' device; returns out [B,gy,gx,C] float32
+    (and the per-cell sample counts [B,gy,gx] when asked)."""
     p = problem_for(x, w, dist, thr, eps, reduction)
-    out = torch.full((p.batch, p.grid_y, p.grid_x, p.channels), float("nan"), dtype=torch.float32,
-                     device=x["image_feats"].device)
+    dev = x["image_feats"].device
+    out = torch.full((p.batch, p.grid_y, p.grid_x, p.channels), float("nan"), dtype=torch.float32, device=dev)
+    cnt = torch.full((p.batch, p.grid_y, p.grid_x), float("nan"), dtype=torch.float32, device=dev) if with_count else None
     st = torch.cuda.current_stream().cuda_stream
     capi.check(capi.forward(p, x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
-                            x["projection_matrices"].data_ptr(), out.data_ptr(), st), "fbev_forward")
+                            x["projection_matrices"].data_ptr(), out.data_ptr(), st,
+                            cnt.data_ptr() if with_count else None), "fbev_forward")
     torch.cuda.synchronize()
-    return out
+    return (out, cnt) if with_count else out
 
 
 def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, want=(True, True),
                   mode="scatter", pair_capacity=None):
     """Backward through the C ABI.  mode "scatter" = fbev_backward, "gather" = fbev_backward_gather
-    with a workspace for `pair_capacity` pairs (default: the worst case)."""
+    with a workspace for `pair_capacity` pairs (default: the worst case), "columns" =
+    fbev_backward_columns overwriting NaN-filled buffers with recounted cell counts,
+    "columns_acc" = the same accumulating into zero-filled buffers with the forward's counts."""
     p = problem_for(x, w, dist, thr, eps, reduction)
     dev = x["image_feats"].device
-    dd = torch.zeros(x["depth_params"].shape, dtype=torch.float32, device=dev) if want[0] else None
-    df = torch.zeros(x["image_feats"].shape, dtype=torch.float32, device=dev) if want[1] else None
+    overwrite = mode in ("columns", "scatter_overwrite", "gather_overwrite")
+    fill = float("nan") if overwrite else 0.0
+    dd = torch.full(x["depth_params"].shape, fill, dtype=torch.float32, device=dev) if want[0] else None
+    df = torch.full(x["image_feats"].shape, fill, dtype=torch.float32, device=dev) if want[1] else None
     st = torch.cuda.current_stream().cuda_stream
     ddp = dd.data_ptr() if dd is not None else None
     dfp = df.data_ptr() if df is not None else None
-    if mode == "scatter":
+    if mode in ("scatter", "scatter_overwrite"):
         capi.check(capi.backward(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
-                                 x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(), ddp, dfp, st),
-                   "fbev_backward")
+                                 x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(), ddp, dfp, st,
+                                 accumulate=not overwrite), "fbev_backward")
+    elif mode in ("columns", "columns_acc"):
+        args = (x["grad_out"].data_ptr(), x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
+                x["projection_matrices"].data_ptr())
+        if mode == "columns":
+            nbytes = capi.backward_columns_workspace_bytes(p)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            capi.check(capi.backward_columns(p, *args, None, ddp, dfp, False, ws.data_ptr(), nbytes, st),
+                       "fbev_backward_columns")
+        else:
+            _, cnt = capi_forward(x, w, dist, thr, eps, reduction, with_count=True)
+            capi.check(capi.backward_columns(p, *args, cnt.data_ptr(), ddp, dfp, True, None, 0, st),
+                       "fbev_backward_columns")
     else:
         cap = capi.backward_max_pairs(p) if pair_capacity is None else pair_capacity
         nbytes = capi.backward_workspace_bytes(p, cap)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         capi.check(capi.backward_gather(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
                                         x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(), ddp, dfp,
-                                        ws.data_ptr(), nbytes, st), "fbev_backward_gather")
+                                        ws.data_ptr(), nbytes, st, accumulate=not overwrite), "fbev_backward_gather")
     torch.cuda.synchronize()
     return dd, df
 

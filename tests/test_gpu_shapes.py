@@ -22,7 +22,7 @@ def small(name="cfg2_surround", **kw):
     return dataclasses.replace(WORKLOADS[name], **kw)
 
 
-def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather"), fwd_tol=(1e-4, 1e-5)):
+def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "columns"), fwd_tol=(1e-4, 1e-5)):
     out = U.capi_forward(x, w, dist, thr).cpu().numpy()
     want = U.oracle_forward(x, w, dist, thr)
     bad, maxabs, ratio = U.violations(out, want, *fwd_tol)
@@ -78,7 +78,7 @@ def test_grid_not_multiple_of_tile_and_unaligned_views():
     shifted.copy_(x["image_feats"])
     assert shifted.data_ptr() % 16 == 4
     y = dict(x, image_feats=shifted)
-    check_all(w, y, 1, modes=("gather",))
+    check_all(w, y, 1, modes=("gather", "columns"))
 
 
 def test_four_by_four_projection_matrices():
@@ -103,7 +103,7 @@ def test_sum_reduction(dist):
     want = U.oracle_forward(x, w, dist, reduce_sum=True)
     assert U.violations(out, want)[0] == 0
     want_dd, want_df = U.oracle_backward(x, w, dist, reduce_sum=True)
-    for mode in ("scatter", "gather"):
+    for mode in ("scatter", "gather", "columns"):
         dd, df = U.capi_backward(x, w, dist, reduction=capi.FBEV_REDUCE_SUM, mode=mode)
         assert U.violations(df.cpu().numpy(), want_df)[0] == 0
         assert U.violations(dd.cpu().numpy(), want_dd)[0] == 0
@@ -135,7 +135,7 @@ def test_degenerate_inputs():
     high = dataclasses.replace(w, roi_range=(-51.2, 51.2, -51.2, 51.2, 500.0, 508.0))
     out = U.capi_forward(x, high, 1)
     assert torch.count_nonzero(out) == 0
-    for mode in ("scatter", "gather"):
+    for mode in ("scatter", "gather", "columns"):
         dd, df = U.capi_backward(x, high, 1, mode=mode)
         assert torch.count_nonzero(dd) == 0 and torch.count_nonzero(df) == 0
     # a threshold nothing passes
@@ -190,7 +190,9 @@ def test_full_size_properties(name, dist):
     assert torch.equal(U.capi_forward(one, w1, dist), out[:1])
     two = dict(x, image_feats=(x["image_feats"] * 2).contiguous())
     assert torch.equal(U.capi_forward(two, w, dist), out * 2)
-    dd, df = U.capi_backward(x, w, dist, mode="gather")
+    dd, df = U.capi_backward(x, w, dist, mode="columns")
+    ddg, dfg = U.capi_backward(x, w, dist, mode="gather")
+    assert torch.allclose(df, dfg, rtol=1e-4, atol=1e-5) and torch.allclose(dd, ddg, rtol=1e-3, atol=1e-4)
     lhs = (out.double() * x["grad_out"].double()).sum().item()
     rhs = (df.double() * x["image_feats"].double()).sum().item()
     assert abs(lhs - rhs) <= 2e-4 * max(abs(lhs), abs(rhs), 1.0), (lhs, rhs)
