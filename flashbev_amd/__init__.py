@@ -7,6 +7,7 @@ Drop-in for the operator layer of yokosyun/FlashBEV's ``flashbevpool`` package
 """
 from .flash_bevpool import FlashBEVPool, flash_bevpool, voxel_geometry
 from .rig import create_projection_matrix
+from .sampling_vt import SamplingVT
 
-__all__ = ["FlashBEVPool", "flash_bevpool", "create_projection_matrix", "voxel_geometry"]
+__all__ = ["FlashBEVPool", "flash_bevpool", "SamplingVT", "create_projection_matrix", "voxel_geometry"]
 __version__ = "0.1.0"

@@ -1,6 +1,6 @@
 """Import-name shim: ``from flashbevpool import flash_bevpool, FlashBEVPool`` resolves to the
 MI355X implementation, so code written against the reference package
 (flashbev/flashbevpool/__init__.py:3-6) runs unchanged."""
-from flashbev_amd import FlashBEVPool, flash_bevpool
+from flashbev_amd import FlashBEVPool, SamplingVT, flash_bevpool
 
-__all__ = ["FlashBEVPool", "flash_bevpool"]
+__all__ = ["FlashBEVPool", "flash_bevpool", "SamplingVT"]
