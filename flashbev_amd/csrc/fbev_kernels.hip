@@ -72,8 +72,9 @@ struct Scope {
 constexpr int kWave = 64;
 constexpr int kWavesPerBlock = 4;
 constexpr int kTile = 8;            // BEV cells are walked in 8x8 tiles for gather locality
-constexpr int kMaxSlotLdsBytes = 12 * 1024;  // per-wave budget for the compacted lists
+constexpr int kMaxSlotLdsBytes = 14 * 1024;  // per-wave budget for the compacted lists
 constexpr int kMaxBlockLdsBytes = 64 * 1024; // dynamic LDS a block may ask for without opting in
+constexpr int kLdsLimitBytes = 150 * 1024;   // what a block may ask for at all (160 KiB per CU)
 constexpr int kXcdCount = 8;                 // accelerator complex dies, each with its own L2
 // The inverse map counts sample corners per texel with integer atomics.  Atomics on one
 // address execute one after the other, and the texels on the horizon collect thousands of
@@ -276,39 +277,134 @@ __device__ __forceinline__ unsigned long long lanemask_lt(int lane) {
     return lane == 0 ? 0ull : (~0ull >> (64 - lane));
 }
 
-// Entry of a compacted list: ENTRY_F4 float4 words.
-//   word 0: forward: corner weights already multiplied by the depth weight
-//           backward: raw bilinear corner weights (w00, w01, w10, w11)
-//   word 1: four texel indices ((b*N+n)*H + v)*W + u as int bits (t00, t01, t10, t11)
-//   word 2 (backward only): wgt, a, b, (k0 | k1 << 16)
-//   word 3 (backward through the inverse map only): for each corner the position of its
-//           (cell, coefficient) pair in the texel-sorted pair array, or -1 if the array is full
-enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2 };
+__device__ __forceinline__ unsigned long long lanemask_le(int lane) { return ~0ull >> (63 - lane); }
 
+// LDS of one block of the cell-centric kernels (float4 units):
+//   [matrices: N*12 floats][decode table: slots*NZ ints]
+//   per wavefront: [16 ints of list lengths][16 float4 of cell centres][slots*NZ ints of
+//   candidates][slots * list_cap entries]
+struct WaveLds {
+    const float *Pm;
+    const int *dec;       // sample index within the wavefront's round -> slot << 28 | camera << 16 | height bin
+    volatile int *cnt;    // entries per slot
+    float4 *cell;         // per slot: x, y, valid flag, ix | iy << 16
+    int *cand;            // samples that survive the cheap test
+    float4 *lst;
+};
+
+__device__ __forceinline__ int lds_p_f4(const KParams &k) { return (k.N * 12 + 3) / 4; }
+__device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots * k.NZ + 3) / 4; }
+
+// Stage the block's matrices and the decode table; returns the wavefront's view.  Ends with a
+// barrier.
+__device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *smem, const float *__restrict__ proj,
+                                                   int b, int entry_f4) {
+    WaveLds L;
+    float *Pm = reinterpret_cast<float *>(smem);
+    int *dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
+    const int dec_f4 = lds_dec_f4(k);
+    const int per_wave_f4 = 4 + 16 + dec_f4 + k.slots * k.list_cap * entry_f4;
+    float4 *wbase = smem + lds_p_f4(k) + dec_f4 + (threadIdx.x >> 6) * per_wave_f4;
+    L.Pm = Pm;
+    L.dec = dec;
+    L.cnt = reinterpret_cast<volatile int *>(wbase);
+    L.cell = wbase + 4;
+    L.cand = reinterpret_cast<int *>(wbase + 20);
+    L.lst = wbase + 20 + dec_f4;
+    for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
+        Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
+    for (int i = threadIdx.x; i < k.slots * k.NZ; i += blockDim.x) {
+        const int slot = i / k.NZ, s = i - slot * k.NZ;
+        const int cam = s / k.gz, iz = s - cam * k.gz;
+        dec[i] = (slot << 28) | (cam << 16) | iz;
+    }
+    __syncthreads();
+    return L;
+}
+
+// Entry of a compacted list: ENTRY_F4 float4 words.
+//   forward   word 0: corner weights already multiplied by the depth weight
+//             word 1: four texel indices ((b*N+n)*H + v)*W + u as int bits (t00, t01, t10, t11)
+//   backward  word 0: du, dv, t00, (u1 != u0) | (v1 != v0) << 1 -- the four weights and texels
+//                     follow from these exactly as phase A computed them
+//             word 1: wgt, a, b, (k0 | k1 << 16)
+//             word 2 (inverse map only): for each corner the position of its (cell, coefficient)
+//                     pair in the texel-sorted pair array, or -1 if the array is full
+enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3 };
+
+// Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
+// pixel coordinate misses the image by more than this fraction, far beyond any rounding of
+// the exact test it would otherwise take (and fail).
+constexpr float kEarlySlack = 1.0e-3f;
+
+// Phase A of one round of a wavefront: the samples of its `slots` cells, in two stages.
+//   stage 1  all slots*NZ samples, lanes = samples: the three dot products and a division-free
+//            test that can only reject samples the exact test rejects too (behind the camera,
+//            or outside the image by more than kEarlySlack).  About 80 % of all samples end
+//            here.  Survivors are compacted, in order, into the candidate list.
+//   stage 2  lanes = candidates, densely packed: the canonical arithmetic (divisions, floor,
+//            bilinear weights), the depth model, the weight threshold; what is kept goes, still
+//            in (camera, height) order, into its slot's entry list.
+// kModeCount writes no entries; it only counts the kept sample corners per (texel, replica).
 template <int ENTRY_F4, typename T, int MODE>
-__device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const T *__restrict__ depth,
-                                        int b, int q0, int lane, float4 *lst, volatile int *cnt,
-                                        const int *__restrict__ chunk_prefix = nullptr,
+__device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, const T *__restrict__ depth, int b, int q0,
+                                        int lane, const int *__restrict__ chunk_prefix = nullptr,
                                         int *__restrict__ cursor = nullptr, int pair_cap = 0) {
-    constexpr bool BACKWARD = MODE != kModeForward;
+    constexpr bool BACKWARD = MODE == kModeScatter || MODE == kModeFill;
     const int total = k.slots * k.NZ;
+    if (lane < 16) L.cnt[lane] = 0;
+    if (lane < k.slots) {
+        int ix = 0, iy = 0;
+        const bool ok = cell_of(k, q0 + lane, ix, iy);
+        L.cell[lane] = make_float4(voxel_coord(k.xmin, ix, k.vx), voxel_coord(k.ymin, iy, k.vy), ok ? 1.0f : 0.0f,
+                                   __int_as_float(ix | (iy << 16)));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- stage 1
+    int n_cand = 0;
+    const float u_max = k.Wi_f * (1.0f + kEarlySlack), v_max = k.Hi_f * (1.0f + kEarlySlack);
     for (int base = 0; base < total; base += kWave) {
-        int idx = base + lane;
-        bool active = idx < total;
-        int slot = active ? idx / k.NZ : k.slots - 1;
-        int s = idx - slot * k.NZ;
-        int cam = s / k.gz;
-        int iz = s - cam * k.gz;
-        int ix, iy;
-        bool ok = active && cell_of(k, q0 + slot, ix, iy);
+        const int idx = base + lane;
+        bool pass = false;
+        if (idx < total) {
+            const int d = L.dec[idx];
+            const float4 c = L.cell[(d >> 28) & 15];
+            if (c.z != 0.0f) {
+                const float *P = L.Pm + ((d >> 16) & 0xfff) * 12;
+                const float x = c.x, y = c.y, z = voxel_coord(k.zmin, d & 0xffff, k.vz);
+                const float D = ((P[8] * x + P[9] * y) + P[10] * z) + P[11];
+                if (D > 0.0f) {
+                    const float U = ((P[0] * x + P[1] * y) + P[2] * z) + P[3];
+                    const float V = ((P[4] * x + P[5] * y) + P[6] * z) + P[7];
+                    const float dc = fmaxf(D, k.eps), lo = -kEarlySlack * dc;
+                    pass = U >= lo && U <= u_max * dc && V >= lo && V <= v_max * dc;
+                }
+            }
+        }
+        const unsigned long long m = __ballot(pass);
+        if (pass) L.cand[n_cand + __popcll(m & lanemask_lt(lane))] = idx;
+        n_cand += __popcll(m);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- stage 2
+    for (int base = 0; base < n_cand; base += kWave) {
+        const int j = base + lane;
+        const bool active = j < n_cand;
+        const int d = active ? L.dec[L.cand[j]] : 0;
+        const int slot = active ? (d >> 28) & 15 : 16 + (lane & 1);   // idle lanes: no real slot
+        const int cam = (d >> 16) & 0xfff;
         float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w2 = w0;
         int4 tx = make_int4(0, 0, 0, 0);
+        int cellxy = 0;
         bool keep = false;
-        if (ok) {
-            float x = voxel_coord(k.xmin, ix, k.vx);
-            float y = voxel_coord(k.ymin, iy, k.vy);
-            float z = voxel_coord(k.zmin, iz, k.vz);
-            Geom g = project_sample(k, Pm + cam * 12, x, y, z);
+        if (active) {
+            const float4 c = L.cell[slot];
+            cellxy = __float_as_int(c.w);
+            Geom g = project_sample(k, L.Pm + cam * 12, c.x, c.y, voxel_coord(k.zmin, d & 0xffff, k.vz));
             if (g.valid) {
                 float w00 = (1.0f - g.du) * (1.0f - g.dv);
                 float w01 = (1.0f - g.du) * g.dv;
@@ -323,29 +419,44 @@ __device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const
                 keep = e.keep;
                 tx = make_int4(t00, t01, t10, t11);
                 if (BACKWARD) {
-                    w0 = make_float4(w00, w01, w10, w11);
+                    w0 = make_float4(g.du, g.dv, __int_as_float(t00),
+                                     __int_as_float((g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0)));
                     w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
                 } else {
                     w0 = make_float4(w00 * e.wgt, w01 * e.wgt, w10 * e.wgt, w11 * e.wgt);
                 }
             }
         }
-        unsigned long long m = __ballot(keep);
-        int lo = max(slot * k.NZ - base, 0);            // first lane of my slot this iteration
-        int hi = min((slot + 1) * k.NZ - base, kWave);   // one past its last lane
-        unsigned long long seg = (~0ull << lo) & (hi >= 64 ? ~0ull : ((1ull << hi) - 1ull));
-        int prefix = __popcll(m & seg & lanemask_lt(lane));
-        int old = cnt[slot];
+        if (MODE == kModeCount) {
+            if (keep) {
+                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
+                atomicAdd(cursor + tx.x * kReplicas + rep, 1);
+                atomicAdd(cursor + tx.y * kReplicas + rep, 1);
+                atomicAdd(cursor + tx.z * kReplicas + rep, 1);
+                atomicAdd(cursor + tx.w * kReplicas + rep, 1);
+            }
+            continue;
+        }
+        // candidates are in sample order, so the lanes of one slot are contiguous: [lo, hi)
+        const int prev_slot = __shfl_up(slot, 1, kWave);
+        const unsigned long long bm = __ballot(lane == 0 || slot != prev_slot);
+        const unsigned long long m = __ballot(keep);
+        const int lo = 63 - __clzll(bm & lanemask_le(lane));
+        const unsigned long long above = lane == 63 ? 0ull : (bm & ~lanemask_le(lane));
+        const int hi = above ? __ffsll((long long)above) - 1 : kWave;
+        const unsigned long long seg = (~0ull << lo) & (hi >= 64 ? ~0ull : ((1ull << hi) - 1ull));
+        const int prefix = __popcll(m & seg & lanemask_lt(lane));
+        const int old = active ? L.cnt[slot] : 0;
         if (keep) {
-            float4 *e = lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
+            float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
             e[0] = w0;
-            e[1] = make_float4(__int_as_float(tx.x), __int_as_float(tx.y), __int_as_float(tx.z),
-                               __int_as_float(tx.w));
-            if (ENTRY_F4 > 2) e[2] = w2;
+            e[1] = BACKWARD ? w2
+                            : make_float4(__int_as_float(tx.x), __int_as_float(tx.y), __int_as_float(tx.z),
+                                          __int_as_float(tx.w));
             if (MODE == kModeFill) {
                 // claim one slot per corner in the texel's segment of the pair array; the four
                 // requests of all lanes are in flight together, so the round trip is paid once
-                const int rep = replica_of(ix, iy);
+                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
                 const int i0 = tx.x * kReplicas + rep, i1 = tx.y * kReplicas + rep;
                 const int i2 = tx.z * kReplicas + rep, i3 = tx.w * kReplicas + rep;
                 int p0 = atomicAdd(cursor + i0, 1);
@@ -364,7 +475,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const float *Pm, const
                                               __int_as_float(p3));
             }
         }
-        if (active && lane == lo) cnt[slot] = old + __popcll(m & seg);
+        if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
     }
 }
 
@@ -380,17 +491,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     const int b = bid / k.blocks_per_batch;
     const int blk = bid - b * k.blocks_per_batch;
 
-    // LDS: [N*12 floats of matrices, padded to float4][per wave: 16 ints of counts][lists]
-    float *Pm = reinterpret_cast<float *>(smem);
-    const int p_f4 = (k.N * 12 + 3) / 4;
-    const int per_wave_f4 = 4 + k.slots * k.list_cap * 2;
-    float4 *wbase = smem + p_f4 + wave * per_wave_f4;
-    volatile int *cnt = reinterpret_cast<volatile int *>(wbase);
-    float4 *lst = wbase + 4;
-
-    for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
-        Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
-    __syncthreads();
+    const WaveLds L = block_lds_setup(k, smem, proj, b, 2);
+    volatile int *cnt = L.cnt;
+    float4 *lst = L.lst;
 
     const int cells_per_wave = k.slots * k.rounds;
     const int slot = lane / k.lanes_per_slot;
@@ -401,8 +504,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     for (int r = 0; r < k.rounds; ++r) {
         const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
-        if (lane < 16) cnt[lane] = 0;
-        phase_a<2, T, kModeForward>(k, Pm, depth, b, q0, lane, lst, cnt);
+        phase_a<2, T, kModeForward>(k, L, depth, b, q0, lane);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
@@ -501,43 +603,26 @@ __global__ __launch_bounds__(256) void fbev_fill_zero_kernel(int *a, long long n
     else if (i < na + nb + nc) c[i - na - nb] = 0;
 }
 
-// One thread per (cell, camera, height) sample: count, per texel, the sample corners that
-// will contribute.  Runs exactly the decisions of phase A (same functions, same inputs).
+// Count, per (texel, replica), the sample corners that will contribute: phase A alone, with
+// exactly the decisions the cell pass takes later (same code, same inputs).
 template <typename T>
-__global__ __launch_bounds__(256) void fbev_count_kernel(KParams k, const T *__restrict__ depth,
-                                                         const float *__restrict__ proj, int *__restrict__ counts,
-                                                         long long total) {
-    long long s = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (s >= total) return;
-    int iz = (int)(s % k.gz);
-    long long r = s / k.gz;
-    int n = (int)(r % k.N); r /= k.N;
-    int ix = (int)(r % k.gx); r /= k.gx;
-    int iy = (int)(r % k.gy);
-    int b = (int)(r / k.gy);
-    const float *P = proj + (size_t)(b * k.N + n) * k.proj_stride;
-    float Pl[12];
-#pragma unroll
-    for (int i = 0; i < 12; ++i) Pl[i] = P[i];
-    Geom g = project_sample(k, Pl, voxel_coord(k.xmin, ix, k.vx), voxel_coord(k.ymin, iy, k.vy),
-                            voxel_coord(k.zmin, iz, k.vz));
-    if (!g.valid) return;
-    float w00 = (1.0f - g.du) * (1.0f - g.dv);
-    float w01 = (1.0f - g.du) * g.dv;
-    float w10 = g.du * (1.0f - g.dv);
-    float w11 = g.du * g.dv;
-    int rowbase = (b * k.N + n) * k.H;
-    int t00 = (rowbase + g.v0) * k.W + g.u0;
-    int t01 = (rowbase + g.v1) * k.W + g.u0;
-    int t10 = (rowbase + g.v0) * k.W + g.u1;
-    int t11 = (rowbase + g.v1) * k.W + g.u1;
-    DepthEval e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
-    if (!e.keep) return;
-    const int rep = replica_of(ix, iy);
-    atomicAdd(counts + t00 * kReplicas + rep, 1);
-    atomicAdd(counts + t01 * kReplicas + rep, 1);
-    atomicAdd(counts + t10 * kReplicas + rep, 1);
-    atomicAdd(counts + t11 * kReplicas + rep, 1);
+__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_count_kernel(KParams k, const T *__restrict__ depth,
+                                                                         const float *__restrict__ proj,
+                                                                         int *__restrict__ counts) {
+    extern __shared__ float4 smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
+    const int b = bid / k.blocks_per_batch;
+    const int blk = bid - b * k.blocks_per_batch;
+    const WaveLds L = block_lds_setup(k, smem, proj, b, 0);
+    const int cells_per_wave = k.slots * k.rounds;
+    for (int r = 0; r < k.rounds; ++r) {
+        const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
+        if (q0 >= k.padded_cells) break;
+        phase_a<0, T, kModeCount>(k, L, depth, b, q0, lane, nullptr, counts, 0);
+        __builtin_amdgcn_wave_barrier();
+    }
 }
 
 // Prefix sum of the counters in two launches.  (1) Every block turns its chunk of 4096
@@ -602,23 +687,16 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
     const int *__restrict__ chunk_prefix, int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap) {
     extern __shared__ float4 smem[];
-    constexpr int EF4 = FILL ? 4 : 3;
+    constexpr int EF4 = FILL ? 3 : 2;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
     const int b = bid / k.blocks_per_batch;
     const int blk = bid - b * k.blocks_per_batch;
 
-    float *Pm = reinterpret_cast<float *>(smem);
-    const int p_f4 = (k.N * 12 + 3) / 4;
-    const int per_wave_f4 = 4 + k.slots * k.list_cap * EF4;
-    float4 *wbase = smem + p_f4 + wave * per_wave_f4;
-    volatile int *cnt = reinterpret_cast<volatile int *>(wbase);
-    float4 *lst = wbase + 4;
-
-    for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
-        Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
-    __syncthreads();
+    const WaveLds L = block_lds_setup(k, smem, proj, b, EF4);
+    volatile int *cnt = L.cnt;
+    float4 *lst = L.lst;
 
     const int cells_per_wave = k.slots * k.rounds;
     const int slot = lane / k.lanes_per_slot;
@@ -633,9 +711,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     for (int r = 0; r < k.rounds; ++r) {
         const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
-        if (lane < 16) cnt[lane] = 0;
-        phase_a<EF4, T, FILL ? kModeFill : kModeScatter>(k, Pm, depth, b, q0, lane, lst, cnt, chunk_prefix, cursor,
-                                                         pair_cap);
+        phase_a<EF4, T, FILL ? kModeFill : kModeScatter>(k, L, depth, b, q0, lane, chunk_prefix, cursor, pair_cap);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
@@ -678,10 +754,17 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 float G = 0.0f;
                 float4 w = make_float4(0.f, 0.f, 0.f, 0.f), tf = w, dw = w, pf = w;
                 if (live) {
-                    w = my[EF4 * e];
-                    tf = my[EF4 * e + 1];
-                    dw = my[EF4 * e + 2];
-                    if (FILL) pf = my[EF4 * e + 3];
+                    const float4 geo = my[EF4 * e];
+                    dw = my[EF4 * e + 1];
+                    if (FILL) pf = my[EF4 * e + 2];
+                    {
+                        const float du = geo.x, dv = geo.y;
+                        w = make_float4((1.0f - du) * (1.0f - dv), (1.0f - du) * dv, du * (1.0f - dv), du * dv);
+                        const int t00 = __float_as_int(geo.z), fl = __float_as_int(geo.w);
+                        const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
+                        tf = make_float4(__int_as_float(t00), __int_as_float(t00 + sv), __int_as_float(t00 + su),
+                                         __int_as_float(t00 + sv + su));
+                    }
                     const size_t o00 = (size_t)__float_as_int(tf.x) * k.C;
                     const size_t o01 = (size_t)__float_as_int(tf.y) * k.C;
                     const size_t o10 = (size_t)__float_as_int(tf.z) * k.C;
@@ -811,26 +894,53 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
         float sa = 0.0f, sb = 0.0f;
-        if (on) {
-#pragma unroll 4
-            for (int e = start + worker; e < end; e += nw) {
-                const float4 pr = *reinterpret_cast<const float4 *>(pairs + e);
-                // a pair is written by the cell pass before this kernel starts; the range check
-                // only keeps a logic error from turning into a wild read
-                if ((unsigned)__float_as_int(pr.x) >= n_cells) continue;
-                const float *row = grad_out + (size_t)__float_as_int(pr.x) * k.C + ch;
-                if (VEC == 1) {
-                    acc[0] = __builtin_fmaf(pr.y, row[0], acc[0]);
-                } else {
-                    const float4 gq = *reinterpret_cast<const float4 *>(row);
-                    acc[0] = __builtin_fmaf(pr.y, gq.x, acc[0]);
-                    acc[1 % VEC] = __builtin_fmaf(pr.y, gq.y, acc[1 % VEC]);
-                    acc[2 % VEC] = __builtin_fmaf(pr.y, gq.z, acc[2 % VEC]);
-                    acc[3 % VEC] = __builtin_fmaf(pr.y, gq.w, acc[3 % VEC]);
+        // A wavefront takes 64 consecutive pairs at a time, one per lane in a single coalesced
+        // load, and hands them to its workers through lane shuffles; four grad_out rows per
+        // worker are in flight before the first is used.  The loop is bound by load latency:
+        // without this the pair load and the row load it addresses form a dependent chain.
+        for (int bstart = start + wave * kWave; bstart < end; bstart += kWavesPerBlock * kWave) {
+            const int nb = min(kWave, end - bstart);
+            float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f);
+            if (lane < nb) pr = *reinterpret_cast<const float4 *>(pairs + bstart + lane);
+            // a pair is written by the cell pass before this kernel starts; the range check
+            // only keeps a logic error from turning into a wild read
+            const bool valid = (unsigned)__float_as_int(pr.x) < n_cells;
+            const int my_cell = valid ? __float_as_int(pr.x) : -1;
+            const float my_coef = valid ? pr.y : 0.0f;
+            if (c0 == 0 && valid) { sa += pr.z; sb += pr.w; }
+            constexpr int UNR = 4;
+            for (int i = 0; i < nb; i += wpw * UNR) {
+                int cells[UNR];
+                float coefs[UNR];
+                float g[UNR][VEC];
+#pragma unroll
+                for (int q = 0; q < UNR; ++q) {
+                    const int j = i + q * wpw + wslot;
+                    const int c = __shfl(my_cell, min(j, kWave - 1), kWave);
+                    coefs[q] = __shfl(my_coef, min(j, kWave - 1), kWave);
+                    cells[q] = (on && j < nb) ? c : -1;
                 }
-                sa += pr.z;
-                sb += pr.w;
+#pragma unroll
+                for (int q = 0; q < UNR; ++q) {
+                    if (cells[q] >= 0) {
+                        const float *row = grad_out + (size_t)cells[q] * k.C + ch;
+                        VecLoad<float, VEC>::ld(row, g[q]);
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < UNR; ++q) {
+                    if (cells[q] >= 0) {
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coefs[q], g[q][v], acc[v]);
+                    }
+                }
             }
+        }
+        // the depth sums sit in the lanes that loaded the pairs: fold them into lane 0
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            sa += __shfl_xor(sa, off, kWave);
+            sb += __shfl_xor(sb, off, kWave);
         }
         __syncthreads();   // previous pass has been read
         if (worker_lane) {
@@ -839,8 +949,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
                 for (int v = 0; v < VEC; ++v) part[worker * stride + lir * VEC + v] = acc[v];
             }
             if (lir == 0) {
-                part[worker * stride + span] = sa;
-                part[worker * stride + span + 1] = sb;
+                part[worker * stride + span] = wslot == 0 ? sa : 0.0f;
+                part[worker * stride + span + 1] = wslot == 0 ? sb : 0.0f;
             }
         }
         __syncthreads();
@@ -1356,7 +1466,7 @@ struct Plan {
     KParams k;
     int vec;        // elements per 16-byte load, or 1
     int cpl;        // channel vectors per lane per pass
-    size_t lds_fwd, lds_bwd, lds_fill;
+    size_t lds_fwd, lds_bwd, lds_fill, lds_count;
 };
 
 int elem_size(int dtype) { return dtype == FBEV_F32 ? 4 : 2; }
@@ -1385,6 +1495,8 @@ int validate(const fbev_problem *p, bool need_channels) {
     const long long nz = (long long)p->num_cams * p->grid_z;
     const long long tiles = (long long)((p->grid_x + kTile - 1) / kTile) * ((p->grid_y + kTile - 1) / kTile);
     if (texels >= (1ll << 31) || nz >= (1 << 20) || tiles * 64 >= (1ll << 30)) return FBEV_ERR_TOO_LARGE;
+    // the sample decode table packs the camera into 12 bits and the height bin into 16
+    if (p->num_cams > 0xfff || p->grid_z > 0xffff) return FBEV_ERR_TOO_LARGE;
     return FBEV_OK;
 }
 
@@ -1417,7 +1529,7 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan) {
     k.lanes_per_slot = lps;
     int slots = kWave / lps;
     // lists of all kernels must fit the per-wave LDS budget (up to 4 float4 per entry in backward)
-    const int entry_bytes = 64;
+    const int entry_bytes = 48 + 4;      // + the candidate index
     while (slots > 1 && (long long)slots * k.NZ * entry_bytes > kMaxSlotLdsBytes) --slots;
     if (slots > 16) slots = 16;
     k.slots = slots;
@@ -1430,11 +1542,25 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan) {
     k.blocks_per_batch = (k.padded_cells + cells_per_block - 1) / cells_per_block;
     k.n_blocks = k.blocks_per_batch * k.B;
     const size_t p_f4 = (size_t)(k.N * 12 + 3) / 4;
-    plan->lds_fwd = (p_f4 + (size_t)kWavesPerBlock * (4 + (size_t)k.slots * k.list_cap * 2)) * 16;
-    plan->lds_bwd = (p_f4 + (size_t)kWavesPerBlock * (4 + (size_t)k.slots * k.list_cap * 3)) * 16;
-    plan->lds_fill = (p_f4 + (size_t)kWavesPerBlock * (4 + (size_t)k.slots * k.list_cap * 4)) * 16;
-    if (plan->lds_fill > (size_t)kMaxBlockLdsBytes) return FBEV_ERR_TOO_LARGE;
+    const size_t dec_f4 = ((size_t)k.slots * k.NZ + 3) / 4;
+    auto block_lds = [&](int entry_f4) {
+        return (p_f4 + dec_f4 + (size_t)kWavesPerBlock * (20 + dec_f4 + (size_t)k.slots * k.list_cap * entry_f4)) * 16;
+    };
+    plan->lds_fwd = block_lds(2);
+    plan->lds_bwd = block_lds(2);
+    plan->lds_fill = block_lds(3);
+    plan->lds_count = block_lds(0);
+    if (plan->lds_fill > (size_t)kLdsLimitBytes) return FBEV_ERR_TOO_LARGE;
     return FBEV_OK;
+}
+
+// More than 64 KiB of dynamic LDS has to be opted into per kernel; only long sample lists
+// (many cameras x height bins) or wide columns get there.
+template <typename Kernel>
+bool lds_opt_in(Kernel kernel, size_t lds) {
+    if (lds <= (size_t)kMaxBlockLdsBytes) return true;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)lds) == hipSuccess;
 }
 
 template <typename T, int VEC>
@@ -1445,9 +1571,12 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
     const T *f = static_cast<const T *>(feats);
     prof::Scope timer(out != nullptr ? prof::kForward : prof::kCellCount, st);
     switch (pl.cpl) {
-        case 1: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 1>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
-        case 2: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 2>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
-        default: hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 4>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
+        case 1: if (!lds_opt_in(fbev_forward_kernel<T, VEC, 1>, pl.lds_fwd)) return FBEV_ERR_LAUNCH;
+                hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 1>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
+        case 2: if (!lds_opt_in(fbev_forward_kernel<T, VEC, 2>, pl.lds_fwd)) return FBEV_ERR_LAUNCH;
+                hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 2>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
+        default: if (!lds_opt_in(fbev_forward_kernel<T, VEC, 4>, pl.lds_fwd)) return FBEV_ERR_LAUNCH;
+                hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 4>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
     }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
@@ -1471,14 +1600,7 @@ template <typename T, int VEC>
 int launch_columns(const Plan &pl, const ColParams &cp, size_t lds, const float *go, const void *depth,
                    const void *feats, const float *proj, const float *count, float *dd, float *df, hipStream_t st) {
     auto kernel = fbev_backward_column_kernel<T, VEC>;
-    // more than 64 KiB of dynamic LDS has to be opted into, once per kernel and size
-    static std::atomic<size_t> opted_in{(size_t)kMaxBlockLdsBytes};
-    if (lds > opted_in.load(std::memory_order_relaxed)) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess)
-            return FBEV_ERR_LAUNCH;
-        opted_in.store(lds, std::memory_order_relaxed);
-    }
+    if (!lds_opt_in(kernel, lds)) return FBEV_ERR_LAUNCH;
     prof::Scope timer(prof::kBackwardColumn, st);
     hipLaunchKernelGGL(kernel, dim3(cp.n_blocks), dim3(kColThreads), lds, st, pl.k, cp, go,
                        static_cast<const T *>(depth), static_cast<const T *>(feats), proj, count, dd, df);
@@ -1494,9 +1616,12 @@ int launch_cells(const Plan &pl, const float *go, const void *depth, const void 
     const size_t lds = FILL ? pl.lds_fill : pl.lds_bwd;
     prof::Scope timer(FILL ? prof::kBackwardCells : prof::kBackwardScatter, st);
     switch (pl.cpl) {
-        case 1: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
-        case 2: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
-        default: hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+        case 1: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 1, FILL>, lds)) return FBEV_ERR_LAUNCH;
+                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+        case 2: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 2, FILL>, lds)) return FBEV_ERR_LAUNCH;
+                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+        default: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 4, FILL>, lds)) return FBEV_ERR_LAUNCH;
+                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
     }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
@@ -1519,10 +1644,11 @@ int dispatch_cells(const fbev_problem *p, const Plan &pl, const float *go, const
 }
 
 template <typename T>
-int launch_count(const Plan &pl, const void *depth, const float *proj, int *counts, long long total, hipStream_t st) {
+int launch_count(const Plan &pl, const void *depth, const float *proj, int *counts, hipStream_t st) {
+    if (!lds_opt_in(fbev_count_kernel<T>, pl.lds_count)) return FBEV_ERR_LAUNCH;
     prof::Scope timer(prof::kCount, st);
-    hipLaunchKernelGGL((fbev_count_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, pl.k,
-                       static_cast<const T *>(depth), proj, counts, total);
+    hipLaunchKernelGGL((fbev_count_kernel<T>), dim3(pl.k.n_blocks), dim3(kWave * kWavesPerBlock), pl.lds_count, st, pl.k,
+                       static_cast<const T *>(depth), proj, counts);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
@@ -1645,7 +1771,7 @@ int fbev_backward_columns(const fbev_problem *p, const float *grad_out, const vo
     const size_t ints = (size_t)kColThreads + kColCells + 2 * kColEntries + 3 * kColMaxRows + 4 + 3 * 64 + kColEntries;
     const size_t lds = 8 * sizeof(float4) + (size_t)kColEntries * 32 + ints * sizeof(int) +
                        (size_t)kColWaves * cp.slots * cp.part_stride * sizeof(float);
-    if (lds > 150 * 1024) return FBEV_ERR_TOO_LARGE;
+    if (lds > (size_t)kLdsLimitBytes) return FBEV_ERR_TOO_LARGE;
     switch (p->in_dtype) {
         case FBEV_F32:
             return pl.vec == 4 ? launch_columns<float, 4>(pl, cp, lds, grad_out, depth, feats, proj, cell_count, d_depth, d_feats, st)
@@ -1691,7 +1817,7 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     hipStream_t st = static_cast<hipStream_t>(stream);
     int *cursor = static_cast<int *>(workspace);
     Pair *pairs = reinterpret_cast<Pair *>(static_cast<char *>(workspace) + index_bytes);
-    const long long texels = texel_count(p), samples = sample_count(p);
+    const long long texels = texel_count(p);
     const long long counters = counter_count(p), chunks = chunk_count(p);
     int *chunk_prefix = cursor + counters;
 
@@ -1699,9 +1825,9 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
                      accumulate ? nullptr : d_feats, texels * p->channels, st);
     if (rc != FBEV_OK) return rc;
     switch (p->in_dtype) {
-        case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, samples, st); break;
-        case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, samples, st); break;
-        default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, samples, st); break;
+        case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, st); break;
+        case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, st); break;
+        default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, st); break;
     }
     if (rc != FBEV_OK) return rc;
     {
