@@ -427,18 +427,39 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                 }
             }
         }
+        const int prev_slot = __shfl_up(slot, 1, kWave);
+        // Consecutive height bins of one (cell, camera) often fall on the same texel (far cells
+        // compress onto the horizon rows).  Corners that repeat the texel of the previous kept
+        // sample of the same cell form a run; when counting, the run's first lane adds the whole
+        // run with ONE atomic.  (Claiming positions per run as well was measured: the shuffles
+        // cost the cell pass more than the saved returning atomics.)
+        int run_lead[4] = {lane, lane, lane, lane}, run_len[4] = {1, 1, 1, 1};
+        if (MODE == kModeCount) {
+            const int prev_keep = __shfl_up((int)keep, 1, kWave);
+            const bool chain = keep && lane > 0 && prev_keep != 0 && prev_slot == slot;
+            const int tc[4] = {tx.x, tx.y, tx.z, tx.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const bool cont = __shfl_up(tc[c], 1, kWave) == tc[c] && chain;
+                const unsigned long long cm = __ballot(cont);
+                // first lane of my run: the highest lane at or below me that does not continue
+                run_lead[c] = 63 - __clzll(~cm & lanemask_le(lane));
+                // lanes after me that continue without a gap
+                const unsigned long long after = lane == 63 ? 0ull : (cm >> (lane + 1));
+                run_len[c] = 1 + (~after == 0ull ? 63 - lane : __ffsll((long long)~after) - 1);
+            }
+        }
         if (MODE == kModeCount) {
             if (keep) {
                 const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
-                atomicAdd(cursor + tx.x * kReplicas + rep, 1);
-                atomicAdd(cursor + tx.y * kReplicas + rep, 1);
-                atomicAdd(cursor + tx.z * kReplicas + rep, 1);
-                atomicAdd(cursor + tx.w * kReplicas + rep, 1);
+                if (run_lead[0] == lane) atomicAdd(cursor + tx.x * kReplicas + rep, run_len[0]);
+                if (run_lead[1] == lane) atomicAdd(cursor + tx.y * kReplicas + rep, run_len[1]);
+                if (run_lead[2] == lane) atomicAdd(cursor + tx.z * kReplicas + rep, run_len[2]);
+                if (run_lead[3] == lane) atomicAdd(cursor + tx.w * kReplicas + rep, run_len[3]);
             }
             continue;
         }
         // candidates are in sample order, so the lanes of one slot are contiguous: [lo, hi)
-        const int prev_slot = __shfl_up(slot, 1, kWave);
         const unsigned long long bm = __ballot(lane == 0 || slot != prev_slot);
         const unsigned long long m = __ballot(keep);
         const int lo = 63 - __clzll(bm & lanemask_le(lane));
@@ -453,27 +474,28 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
             e[1] = BACKWARD ? w2
                             : make_float4(__int_as_float(tx.x), __int_as_float(tx.y), __int_as_float(tx.z),
                                           __int_as_float(tx.w));
-            if (MODE == kModeFill) {
-                // claim one slot per corner in the texel's segment of the pair array; the four
-                // requests of all lanes are in flight together, so the round trip is paid once
-                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
-                const int i0 = tx.x * kReplicas + rep, i1 = tx.y * kReplicas + rep;
-                const int i2 = tx.z * kReplicas + rep, i3 = tx.w * kReplicas + rep;
-                int p0 = atomicAdd(cursor + i0, 1);
-                int p1 = atomicAdd(cursor + i1, 1);
-                int p2 = atomicAdd(cursor + i2, 1);
-                int p3 = atomicAdd(cursor + i3, 1);
-                p0 += chunk_prefix[i0 >> kScanChunkBits];
-                p1 += chunk_prefix[i1 >> kScanChunkBits];
-                p2 += chunk_prefix[i2 >> kScanChunkBits];
-                p3 += chunk_prefix[i3 >> kScanChunkBits];
-                p0 = p0 < pair_cap ? p0 : -1;
-                p1 = p1 < pair_cap ? p1 : -1;
-                p2 = p2 < pair_cap ? p2 : -1;
-                p3 = p3 < pair_cap ? p3 : -1;
-                e[ENTRY_F4 - 1] = make_float4(__int_as_float(p0), __int_as_float(p1), __int_as_float(p2),
-                                              __int_as_float(p3));
-            }
+        }
+        if (MODE == kModeFill && keep) {
+            // claim one position per corner in the texel's segment of the pair array; the four
+            // requests of all lanes are in flight together, so the round trip is paid once
+            const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
+            const int i0 = tx.x * kReplicas + rep, i1 = tx.y * kReplicas + rep;
+            const int i2 = tx.z * kReplicas + rep, i3 = tx.w * kReplicas + rep;
+            int p0 = atomicAdd(cursor + i0, 1);
+            int p1 = atomicAdd(cursor + i1, 1);
+            int p2 = atomicAdd(cursor + i2, 1);
+            int p3 = atomicAdd(cursor + i3, 1);
+            p0 += chunk_prefix[i0 >> kScanChunkBits];
+            p1 += chunk_prefix[i1 >> kScanChunkBits];
+            p2 += chunk_prefix[i2 >> kScanChunkBits];
+            p3 += chunk_prefix[i3 >> kScanChunkBits];
+            p0 = p0 < pair_cap ? p0 : -1;
+            p1 = p1 < pair_cap ? p1 : -1;
+            p2 = p2 < pair_cap ? p2 : -1;
+            p3 = p3 < pair_cap ? p3 : -1;
+            float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
+            e[ENTRY_F4 - 1] = make_float4(__int_as_float(p0), __int_as_float(p1), __int_as_float(p2),
+                                          __int_as_float(p3));
         }
         if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
     }
