@@ -40,6 +40,13 @@ from flashbev_amd.flash_bevpool import voxel_geometry  # noqa: E402
 from flashbev_amd.workloads import WORKLOADS, algorithmic_bytes, make_inputs  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
+# counters read for a 256 MiB copy (x2.000 / x1.000); see profiles/.  Only for the workload
+# and kernels the counters were collected on; anything else reports null.
+MEASURED_TRAFFIC = {
+    ("cfg2_surround", "laplace", 0): {"backward": 57.1e6, "forward": 8.39e6,
+                                      "source": "profiles/cfg2_surround_laplace_fwd_bwd_gather.md"},
+}
 DIST_OF = {"gaussian": (0, "parametric"), "laplace": (1, "parametric"), "categorical": (2, "categorical")}
 
 
@@ -232,6 +239,7 @@ def main():
     k_ms, k_bytes, k_names = (bwd_k_ms, bb, bwd_names) if dominant == "backward" else (fwd_k_ms, fb, fwd_names)
     achieved = k_bytes / k_ms / 1e6  # GB/s
     top = max(kernels, key=lambda k: kernels[k]["mean_us"] * kernels[k]["calls_per_step"])
+    traffic = MEASURED_TRAFFIC.get((w.name, args.depth, args.backward_mode))
     line = {
         "metric": "BEV-pool fwd+bwd latency (ms) & effective HBM GB/s, 6 cams 128x128xZ=8, 1 GPU",
         "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -248,7 +256,8 @@ def main():
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": f"{dominant} pass = " + " + ".join(k_names),
                      "dominant_kernel": top, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": k_bytes,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic[dominant] if traffic else None,
+                     "traffic_source": traffic["source"] if traffic else None, "algorithmic_bytes": k_bytes,
                      "kernel_ms": k_ms,
                      "forward": {"algorithmic_bytes": fb, "kernel_ms": fwd_k_ms,
                                  "frac": fb / fwd_k_ms / 1e6 / HBM_PEAK_GBS if fwd_k_ms else None}},
