@@ -832,31 +832,56 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                     }
                 }
                 if (live && lis == 0) {
-                    const int kk = __float_as_int(dw.w);
-                    const int k0 = kk & 0xffff, k1 = kk >> 16;
-                    const float ga = G * dw.y, gb = G * dw.z;
-                    const int t[4] = {__float_as_int(tf.x), __float_as_int(tf.y), __float_as_int(tf.z),
-                                      __float_as_int(tf.w)};
-                    const float wc[4] = {w.x, w.y, w.z, w.w};
-                    const int pos[4] = {__float_as_int(pf.x), __float_as_int(pf.y), __float_as_int(pf.z),
-                                        __float_as_int(pf.w)};
+                    if (FILL && first_pass && parametric) {
+                        // the pairs are written after the loop, 64 at a time; keep G with the entry
+                        // (the bin word of a parametric entry is unused)
+                        if (need_G) const_cast<float4 *>(my)[EF4 * e + 1].w = G;
+                    } else if (need_G) {
+                        // scatter path, categorical bins, or a later channel pass whose share of G
+                        // cannot be folded into a pair already written
+                        const int kk = __float_as_int(dw.w);
+                        const int k0 = kk & 0xffff, k1 = kk >> 16;
+                        const float ga = G * dw.y, gb = G * dw.z;
+                        const int t[4] = {__float_as_int(tf.x), __float_as_int(tf.y), __float_as_int(tf.z),
+                                          __float_as_int(tf.w)};
+                        const float wc[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const bool paired = FILL && pos[c] >= 0;
-                        if (paired && first_pass) {
-                            // G of a later channel pass cannot be folded into a pair already written:
-                            // passes after the first add their share of the depth gradient atomically.
-                            Pair pr;
-                            pr.cell = cell;
-                            pr.coef = wc[c] * dw.x * inv;
-                            pr.da = (need_G && parametric) ? ga * wc[c] : 0.0f;
-                            pr.db = (need_G && parametric) ? gb * wc[c] : 0.0f;
-                            *reinterpret_cast<float4 *>(pairs + pos[c]) =
-                                make_float4(__int_as_float(pr.cell), pr.coef, pr.da, pr.db);
-                        }
-                        if (need_G && !(paired && first_pass && parametric)) {
+                        for (int c = 0; c < 4; ++c) {
                             atomic_add_f32(d_depth + (size_t)t[c] * Dd + k0, ga * wc[c]);
                             atomic_add_f32(d_depth + (size_t)t[c] * Dd + k1, gb * wc[c]);
+                        }
+                    }
+                }
+            }
+            if (FILL && first_pass) {
+                // ---- the pairs of this round: lanes = (entry, corner), every slot in turn
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                for (int sl = 0; sl < k.slots; ++sl) {
+                    const int ns = cnt[sl];
+                    if (ns == 0) continue;
+                    const int cxy = __float_as_int(L.cell[sl].w);
+                    const int pcell = (b * k.gy + (cxy >> 16)) * k.gx + (cxy & 0xffff);
+                    const float pinv = k.reduce_sum ? 1.0f : 1.0f / (float)ns;
+                    const float4 *lst_s = lst + (size_t)sl * k.list_cap * EF4;
+                    for (int i = lane; i < ns * 4; i += kWave) {
+                        const int pe = i >> 2, c = i & 3;
+                        const float4 geo = lst_s[EF4 * pe], dwp = lst_s[EF4 * pe + 1], pfp = lst_s[EF4 * pe + 2];
+                        const float du = geo.x, dv = geo.y;
+                        // corner c: 0 (v0,u0) 1 (v1,u0) 2 (v0,u1) 3 (v1,u1); same products as phase A
+                        const float wu = (c & 2) ? du : 1.0f - du, wv = (c & 1) ? dv : 1.0f - dv;
+                        const float wcc = wu * wv;
+                        const int posc = __float_as_int(c == 0 ? pfp.x : (c == 1 ? pfp.y : (c == 2 ? pfp.z : pfp.w)));
+                        const float Gp = (need_G && parametric) ? dwp.w : 0.0f;   // already carries 1/count
+                        const float da = Gp * dwp.y * wcc, db = Gp * dwp.z * wcc;
+                        if (posc >= 0) {
+                            *reinterpret_cast<float4 *>(pairs + posc) =
+                                make_float4(__int_as_float(pcell), wcc * dwp.x * pinv, da, db);
+                        } else if (need_G && parametric) {
+                            const int fl = __float_as_int(geo.w);
+                            const int tt = __float_as_int(geo.z) + ((c & 1) && (fl & 2) ? k.W : 0) + ((c & 2) ? (fl & 1) : 0);
+                            atomic_add_f32(d_depth + (size_t)tt * 2, da);
+                            atomic_add_f32(d_depth + (size_t)tt * 2 + 1, db);
                         }
                     }
                 }
