@@ -273,6 +273,15 @@ __device__ __forceinline__ int xcd_swizzle(int bid, int n_blocks) {
 
 __device__ __forceinline__ int replica_of(int ix, int iy) { return (ix + 5 * iy) & (kReplicas - 1); }
 
+// Value of the lane whose index differs in bit 0 (bit 1) inside every group of four lanes.
+// All 64 lanes must be active.
+__device__ __forceinline__ float quad_xor1(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ float quad_xor2(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+}
+
 __device__ __forceinline__ unsigned long long lanemask_lt(int lane) {
     return lane == 0 ? 0ull : (~0ull >> (64 - lane));
 }
@@ -651,50 +660,71 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_count_kernel(KPara
 // counters into exclusive prefix sums within the chunk and records the chunk total.
 // (2) One block turns the chunk totals into exclusive prefix sums.  A counter's global
 // position is chunk_prefix[i >> 12] + v[i]; nobody needs it materialised.
+// (One launch with a last-block-done ticket was measured: the device-scope release every block
+// then needs costs more than the second launch.)
+
+// Inclusive scan of one value per thread of a 1024-thread block: shuffles inside a wavefront,
+// LDS (32 ints) across the 16 wavefronts.
+__device__ __forceinline__ int block_scan_1024(int *part, int tid, int sum) {
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
+    int incl = sum;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const int other = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += other;
+    }
+    if (lane == kWave - 1) part[wave] = incl;
+    __syncthreads();
+    if (tid < 16) {
+        int t = part[tid];
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+            const int other = __shfl_up(t, off, kWave);
+            if (tid >= off) t += other;
+        }
+        part[16 + tid] = t;
+    }
+    __syncthreads();
+    return incl + (wave == 0 ? 0 : part[16 + wave - 1]);
+}
+
 __global__ __launch_bounds__(1024) void fbev_scan_chunks_kernel(int *__restrict__ v, long long n,
                                                                 int *__restrict__ chunk_sums) {
-    __shared__ int part[1024];
+    __shared__ int part[32];
     const int tid = threadIdx.x;
     const long long base = ((long long)blockIdx.x << kScanChunkBits) + tid * 4;
-    int c[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) c[j] = base + j < n ? v[base + j] : 0;
-    const int sum = c[0] + c[1] + c[2] + c[3];
-    part[tid] = sum;
-    __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        int add = tid >= off ? part[tid - off] : 0;
-        __syncthreads();
-        part[tid] += add;
-        __syncthreads();
+    int4 c = make_int4(0, 0, 0, 0);
+    if (base + 3 < n) {
+        c = *reinterpret_cast<const int4 *>(v + base);
+    } else {
+        if (base < n) c.x = v[base];
+        if (base + 1 < n) c.y = v[base + 1];
+        if (base + 2 < n) c.z = v[base + 2];
     }
-    int run = part[tid] - sum;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (base + j < n) v[base + j] = run;
-        run += c[j];
+    const int sum = c.x + c.y + c.z + c.w;
+    const int incl = block_scan_1024(part, tid, sum);
+    const int run = incl - sum;
+    const int4 o = make_int4(run, run + c.x, run + c.x + c.y, run + c.x + c.y + c.z);
+    if (base + 3 < n) {
+        *reinterpret_cast<int4 *>(v + base) = o;
+    } else {
+        if (base < n) v[base] = o.x;
+        if (base + 1 < n) v[base + 1] = o.y;
+        if (base + 2 < n) v[base + 2] = o.z;
     }
-    if (tid == 1023) chunk_sums[blockIdx.x] = part[1023];
+    if (tid == 1023) chunk_sums[blockIdx.x] = incl;
 }
 
 __global__ __launch_bounds__(1024) void fbev_scan_sums_kernel(int *v, int n) {
-    __shared__ int part[1024];
+    __shared__ int part[32];
     const int tid = threadIdx.x;
-    const int chunk = (n + 1023) / 1024;
-    const int lo = min(tid * chunk, n), hi = min(lo + chunk, n);
+    const int per = (n + 1023) / 1024;
+    const int lo = min(tid * per, n), hi = min(lo + per, n);
     int sum = 0;
     for (int i = lo; i < hi; ++i) sum += v[i];
-    part[tid] = sum;
-    __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        int add = tid >= off ? part[tid - off] : 0;
-        __syncthreads();
-        part[tid] += add;
-        __syncthreads();
-    }
-    int run = part[tid] - sum;
+    int run = block_scan_1024(part, tid, sum) - sum;
     for (int i = lo; i < hi; ++i) {
-        int c = v[i];
+        const int c = v[i];
         v[i] = run;
         run += c;
     }
@@ -730,126 +760,169 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     // the inner product <grad_out, sampled feature> is only needed for the depth gradient
     const bool need_G = d_depth != nullptr;
 
+    // G of four entries is summed over the lanes of a slot at a time when the slots start on
+    // multiples of four lanes (always, on the 128-bit path)
+    const bool grouped = (k.lanes_per_slot & 3) == 0;
+
     for (int r = 0; r < k.rounds; ++r) {
         const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
+        int ix = 0, iy = 0;
+        const bool mine = carrier && cell_of(k, q0 + slot, ix, iy);
+        const int cell = (b * k.gy + iy) * k.gx + ix;
+        const float *go = grad_out + (size_t)cell * k.C;
+        // the cell's grad_out row (first channel pass) is requested before phase A and arrives
+        // while the samples are evaluated
+        float g[CPL][VEC];
+        auto load_g = [&](int c0) {
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+                const int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) g[j][v] = 0.0f;
+                if (mine && ch < k.C) {
+                    if (VEC == 1) {
+                        g[j][0] = go[ch];
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < VEC; v += 4) {
+                            const float4 t = *reinterpret_cast<const float4 *>(go + ch + v);
+                            g[j][v] = t.x; g[j][v + 1] = t.y; g[j][v + 2] = t.z; g[j][v + 3] = t.w;
+                        }
+                    }
+                }
+            }
+        };
+        load_g(0);
         phase_a<EF4, T, FILL ? kModeFill : kModeScatter>(k, L, depth, b, q0, lane, chunk_prefix, cursor, pair_cap);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
-        int ix = 0, iy = 0;
-        bool mine = carrier && cell_of(k, q0 + slot, ix, iy);
         const int n = mine ? cnt[slot] : 0;
         // every lane of the wavefront takes part in the shuffles below, so all lanes run
         // the longest list of the wavefront and idle past their own.
         int n_max = n;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) n_max = max(n_max, __shfl_xor(n_max, off, kWave));
-        const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * EF4;
-        const int cell = (b * k.gy + iy) * k.gx + ix;
-        const float *go = grad_out + (size_t)cell * k.C;
+        float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * EF4;
         const float inv = (k.reduce_sum || n == 0) ? 1.0f : 1.0f / (float)n;
 
         for (int c0 = 0; c0 < k.C; c0 += span) {
             const bool first_pass = c0 == 0;
-            float g[CPL][VEC];
+            if (!first_pass) load_g(c0);
 #pragma unroll
-            for (int j = 0; j < CPL; ++j) {
-                int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
+            for (int j = 0; j < CPL; ++j)
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) g[j][v] = 0.0f;
-                if (mine && n > 0 && ch < k.C) {
-                    if (VEC == 1) {
-                        g[j][0] = go[ch] * inv;
-                    } else {
-#pragma unroll
-                        for (int v = 0; v < VEC; v += 4) {
-                            float4 t = *reinterpret_cast<const float4 *>(go + ch + v);
-                            g[j][v] = t.x * inv; g[j][v + 1] = t.y * inv;
-                            g[j][v + 2] = t.z * inv; g[j][v + 3] = t.w * inv;
-                        }
-                    }
-                }
-            }
-            for (int e = 0; e < n_max; ++e) {
-                const bool live = e < n;
+                for (int v = 0; v < VEC; ++v) g[j][v] = n > 0 ? g[j][v] * inv : 0.0f;
+
+            // this lane's share of <grad_out, sampled feature> of entry e (e < n); on the scatter
+            // path (and for corners without room in the pair array) also the feature-gradient atomics
+            auto entry_share = [&](int e) -> float {
                 float G = 0.0f;
-                float4 w = make_float4(0.f, 0.f, 0.f, 0.f), tf = w, dw = w, pf = w;
-                if (live) {
-                    const float4 geo = my[EF4 * e];
-                    dw = my[EF4 * e + 1];
-                    if (FILL) pf = my[EF4 * e + 2];
-                    {
-                        const float du = geo.x, dv = geo.y;
-                        w = make_float4((1.0f - du) * (1.0f - dv), (1.0f - du) * dv, du * (1.0f - dv), du * dv);
-                        const int t00 = __float_as_int(geo.z), fl = __float_as_int(geo.w);
-                        const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
-                        tf = make_float4(__int_as_float(t00), __int_as_float(t00 + sv), __int_as_float(t00 + su),
-                                         __int_as_float(t00 + sv + su));
-                    }
-                    const size_t o00 = (size_t)__float_as_int(tf.x) * k.C;
-                    const size_t o01 = (size_t)__float_as_int(tf.y) * k.C;
-                    const size_t o10 = (size_t)__float_as_int(tf.z) * k.C;
-                    const size_t o11 = (size_t)__float_as_int(tf.w) * k.C;
-                    const float a00 = w.x * dw.x, a01 = w.y * dw.x, a10 = w.z * dw.x, a11 = w.w * dw.x;
-                    // corners whose pair found no room in the pair array fall back to atomics
-                    const bool s00 = !FILL || __float_as_int(pf.x) < 0, s01 = !FILL || __float_as_int(pf.y) < 0;
-                    const bool s10 = !FILL || __float_as_int(pf.z) < 0, s11 = !FILL || __float_as_int(pf.w) < 0;
+                const float4 geo = my[EF4 * e];
+                const float wgt = my[EF4 * e + 1].x;
+                const float du = geo.x, dv = geo.y;
+                const float w00 = (1.0f - du) * (1.0f - dv), w01 = (1.0f - du) * dv, w10 = du * (1.0f - dv), w11 = du * dv;
+                const int t00 = __float_as_int(geo.z), fl = __float_as_int(geo.w);
+                const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
+                const size_t o00 = (size_t)t00 * k.C, o01 = (size_t)(t00 + sv) * k.C;
+                const size_t o10 = (size_t)(t00 + su) * k.C, o11 = (size_t)(t00 + sv + su) * k.C;
+                bool s00 = true, s01 = true, s10 = true, s11 = true;
+                if (FILL) {
+                    const float4 pf = my[EF4 * e + 2];
+                    s00 = __float_as_int(pf.x) < 0; s01 = __float_as_int(pf.y) < 0;
+                    s10 = __float_as_int(pf.z) < 0; s11 = __float_as_int(pf.w) < 0;
+                }
+                const float a00 = w00 * wgt, a01 = w01 * wgt, a10 = w10 * wgt, a11 = w11 * wgt;
 #pragma unroll
-                    for (int j = 0; j < CPL; ++j) {
-                        int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
-                        if (ch < k.C) {
-                            if (need_G) {
-                                float f00[VEC], f01[VEC], f10[VEC], f11[VEC];
-                                VecLoad<T, VEC>::ld(feats + o00 + ch, f00);
-                                VecLoad<T, VEC>::ld(feats + o01 + ch, f01);
-                                VecLoad<T, VEC>::ld(feats + o10 + ch, f10);
-                                VecLoad<T, VEC>::ld(feats + o11 + ch, f11);
+                for (int j = 0; j < CPL; ++j) {
+                    const int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
+                    if (ch < k.C) {
+                        if (need_G) {
+                            float f00[VEC], f01[VEC], f10[VEC], f11[VEC];
+                            VecLoad<T, VEC>::ld(feats + o00 + ch, f00);
+                            VecLoad<T, VEC>::ld(feats + o01 + ch, f01);
+                            VecLoad<T, VEC>::ld(feats + o10 + ch, f10);
+                            VecLoad<T, VEC>::ld(feats + o11 + ch, f11);
 #pragma unroll
-                                for (int v = 0; v < VEC; ++v) {
-                                    float f = bilerp(w.x, w.y, w.z, w.w, f00[v], f01[v], f10[v], f11[v]);
-                                    G = __builtin_fmaf(g[j][v], f, G);
-                                }
+                            for (int v = 0; v < VEC; ++v) {
+                                const float f = __builtin_fmaf(w11, f11[v], __builtin_fmaf(w10, f10[v],
+                                                __builtin_fmaf(w01, f01[v], w00 * f00[v])));
+                                G = __builtin_fmaf(g[j][v], f, G);
                             }
-                            if (d_feats != nullptr) {
+                        }
+                        if (d_feats != nullptr && (s00 || s01 || s10 || s11)) {
 #pragma unroll
-                                for (int v = 0; v < VEC; ++v) {
-                                    if (s00) atomic_add_f32(d_feats + o00 + ch + v, g[j][v] * a00);
-                                    if (s01) atomic_add_f32(d_feats + o01 + ch + v, g[j][v] * a01);
-                                    if (s10) atomic_add_f32(d_feats + o10 + ch + v, g[j][v] * a10);
-                                    if (s11) atomic_add_f32(d_feats + o11 + ch + v, g[j][v] * a11);
-                                }
+                            for (int v = 0; v < VEC; ++v) {
+                                if (s00) atomic_add_f32(d_feats + o00 + ch + v, g[j][v] * a00);
+                                if (s01) atomic_add_f32(d_feats + o01 + ch + v, g[j][v] * a01);
+                                if (s10) atomic_add_f32(d_feats + o10 + ch + v, g[j][v] * a10);
+                                if (s11) atomic_add_f32(d_feats + o11 + ch + v, g[j][v] * a11);
                             }
                         }
                     }
                 }
-                if (need_G) {
-                    // sum G over the lanes of the slot: lane `lis` adds lane `lis + off`
+                return G;
+            };
+            // what one lane does with the complete G of entry e
+            auto entry_done = [&](int e, float G) {
+                if (FILL && first_pass && parametric) {
+                    // the pairs are written after the loop, 64 at a time; keep G with the entry
+                    // (the bin word of a parametric entry is unused)
+                    my[EF4 * e + 1].w = G;
+                } else {
+                    // scatter path, categorical bins, or a later channel pass whose share of G
+                    // cannot be folded into a pair already written
+                    const float4 geo = my[EF4 * e], dw = my[EF4 * e + 1];
+                    const float du = geo.x, dv = geo.y;
+                    const float wc[4] = {(1.0f - du) * (1.0f - dv), (1.0f - du) * dv, du * (1.0f - dv), du * dv};
+                    const int t00 = __float_as_int(geo.z), fl = __float_as_int(geo.w);
+                    const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
+                    const int t[4] = {t00, t00 + sv, t00 + su, t00 + sv + su};
+                    const int kk = __float_as_int(dw.w);
+                    const int k0 = parametric ? 0 : (kk & 0xffff), k1 = parametric ? 1 : (kk >> 16);
+                    const float ga = G * dw.y, gb = G * dw.z;
 #pragma unroll
-                    for (int off = 32; off > 0; off >>= 1) {
-                        float other = __shfl_down(G, off, kWave);
-                        if (lis + off < k.lanes_per_slot) G += other;
+                    for (int c = 0; c < 4; ++c) {
+                        atomic_add_f32(d_depth + (size_t)t[c] * Dd + k0, ga * wc[c]);
+                        atomic_add_f32(d_depth + (size_t)t[c] * Dd + k1, gb * wc[c]);
                     }
                 }
-                if (live && lis == 0) {
-                    if (FILL && first_pass && parametric) {
-                        // the pairs are written after the loop, 64 at a time; keep G with the entry
-                        // (the bin word of a parametric entry is unused)
-                        if (need_G) const_cast<float4 *>(my)[EF4 * e + 1].w = G;
-                    } else if (need_G) {
-                        // scatter path, categorical bins, or a later channel pass whose share of G
-                        // cannot be folded into a pair already written
-                        const int kk = __float_as_int(dw.w);
-                        const int k0 = kk & 0xffff, k1 = kk >> 16;
-                        const float ga = G * dw.y, gb = G * dw.z;
-                        const int t[4] = {__float_as_int(tf.x), __float_as_int(tf.y), __float_as_int(tf.z),
-                                          __float_as_int(tf.w)};
-                        const float wc[4] = {w.x, w.y, w.z, w.w};
+            };
+
+            if (grouped) {
+                for (int e0 = 0; e0 < n_max; e0 += 4) {
+                    float G0 = e0 < n ? entry_share(e0) : 0.0f;
+                    float G1 = e0 + 1 < n ? entry_share(e0 + 1) : 0.0f;
+                    float G2 = e0 + 2 < n ? entry_share(e0 + 2) : 0.0f;
+                    float G3 = e0 + 3 < n ? entry_share(e0 + 3) : 0.0f;
+                    if (need_G) {
+                        // two exchange steps inside every group of four lanes leave lane q of the
+                        // group with the group's sum for entry (q & 1) * 2 + (q >> 1) ...
+                        const bool b0 = lane & 1, b1 = lane & 2;
+                        const float ra = quad_xor1(b0 ? G0 : G2), rb = quad_xor1(b0 ? G1 : G3);
+                        const float ka = (b0 ? G2 : G0) + ra, kb = (b0 ? G3 : G1) + rb;
+                        float Gq = (b1 ? kb : ka) + quad_xor2(b1 ? ka : kb);
+                        // ... and four more add up the groups of the slot
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) {
-                            atomic_add_f32(d_depth + (size_t)t[c] * Dd + k0, ga * wc[c]);
-                            atomic_add_f32(d_depth + (size_t)t[c] * Dd + k1, gb * wc[c]);
+                        for (int off = 32; off >= 4; off >>= 1) {
+                            const float other = __shfl_down(Gq, off, kWave);
+                            if (lis + off < k.lanes_per_slot) Gq += other;
                         }
+                        const int e = e0 + ((lis & 1) << 1) + ((lis >> 1) & 1);
+                        if (lis < 4 && e < n) entry_done(e, Gq);
+                    }
+                }
+            } else {
+                for (int e = 0; e < n_max; ++e) {
+                    float G = e < n ? entry_share(e) : 0.0f;
+                    if (need_G) {
+#pragma unroll
+                        for (int off = 32; off > 0; off >>= 1) {
+                            const float other = __shfl_down(G, off, kWave);
+                            if (lis + off < k.lanes_per_slot) G += other;
+                        }
+                        if (e < n && lis == 0) entry_done(e, G);
                     }
                 }
             }
