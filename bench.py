@@ -8,7 +8,10 @@ per-cell sample counts) and the backward kernels (whose first launch zero-fills 
 gradient buffers), all queued on PyTorch's current stream through the extension module.  The default workload is the 6-camera 128x128x8 fp32 configuration
 (``cfg2_surround``) with the reference benchmark's depth model (per-pixel Laplace
 parameters, tools/config/config.yaml:29).  The single JSON line printed on stdout carries
-  value / ms_per_step   forward+backward latency per step (ms)
+  value / ms_per_step   forward+backward latency per step (ms), K eagerly queued steps between two
+                        synchronisations; ms_per_step_graph is the same step captured into a HIP
+                        graph and replayed K times (checked against the eager result first) --
+                        on this machine the eager queue is already GPU-bound and no slower
   roofline              the dominant pass (the backward, five kernel launches): its compulsory
                         bytes / the summed mean durations of its kernels, measured with HIP
                         events the library records around every one of its launches over a
@@ -87,15 +90,23 @@ class Runner:
 
 
 def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
-    """Wall-clock over exactly `steps` steps plus per-kernel HIP-event durations."""
-    for _ in range(warmup):
+    """Wall-clock over exactly `steps` eagerly queued steps (nothing but the operator's launches
+    between the two synchronisations), then the same steps again with events around each pass
+    for the forward / backward split."""
+    def step():
         r.forward()
         if with_backward:
             r.backward()
-    torch.cuda.synchronize()
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+
+    for _ in range(warmup):
+        step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
     for i in range(steps):
         ev[i][0].record()
         r.forward()
@@ -105,10 +116,49 @@ def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
             r.backward()
             ev[i][3].record()
     torch.cuda.synchronize()
-    t1 = time.perf_counter()
     fwd = [ev[i][0].elapsed_time(ev[i][1]) for i in range(steps)]
     bwd = [ev[i][2].elapsed_time(ev[i][3]) for i in range(steps)] if with_backward else []
     return (t1 - t0) * 1e3 / steps, fwd, bwd
+
+
+def time_graph_steps(r: Runner, steps: int, warmup: int):
+    """One step captured into a HIP graph and replayed: the same kernels on the same buffers,
+    submitted with one call per step.  Returns ms per step, or None when capture fails.  The
+    replayed gradients are checked against the eager ones before anything is timed."""
+    r.forward()
+    r.backward()
+    torch.cuda.synchronize()
+    want = (r.out.clone(), r.d_depth.clone(), r.d_feats.clone())
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            r.forward()
+            r.backward()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            r.forward()
+            r.backward()
+    except Exception as exc:  # pragma: no cover - depends on the runtime
+        print(f"bench.py: graph capture failed ({exc}); reporting the eager timing", file=sys.stderr)
+        return None
+    for i in range(max(3, warmup)):
+        if i < 3:
+            r.out.zero_(); r.d_depth.fill_(7.0); r.d_feats.fill_(7.0)
+        graph.replay()
+        if i < 3:
+            torch.cuda.synchronize()
+            for got, ref, what in zip((r.out, r.d_depth, r.d_feats), want, ("out", "d_depth", "d_feats")):
+                if not torch.allclose(got, ref, rtol=1e-4, atol=1e-5):
+                    raise RuntimeError(f"graph replay {i}: {what} differs from the eager result")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps
 
 
 def profile_steps(r: Runner, steps: int):
@@ -202,6 +252,7 @@ def main():
     ap.add_argument("--depth", default="laplace", choices=sorted(DIST_OF))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--table", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eagerly queued steps only")
     ap.add_argument("--backward-mode", type=int, default=0, choices=(0, 1, 2, 3),
                     help="0 auto (default), 1 atomic scatter, 2 inverse-map gather, 3 column owner")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
@@ -227,7 +278,9 @@ def main():
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n}))
         return
     r = Runner(w, args.depth, backward_mode=args.backward_mode)
-    ms, fwd, bwd = time_steps(r, args.steps, args.warmup, True)
+    eager_ms, fwd, bwd = time_steps(r, args.steps, args.warmup, True)
+    graph_ms = None if args.no_graph else time_graph_steps(r, args.steps, args.warmup)
+    ms = eager_ms
     kernels = profile_steps(r, args.steps)
     fwd_ms, bwd_ms = statistics.mean(fwd), statistics.mean(bwd)
     fb, bb = algorithmic_bytes(w, r.model, False), algorithmic_bytes(w, r.model, True)
@@ -249,7 +302,9 @@ def main():
         "config": {"workload": w.name, "depth_model": args.depth, "batch": w.batch, "cams": w.num_cams,
                    "channels": w.channels, "feat_hw": list(w.feat_hw), "grid": list(w.grid_size),
                    "backward": {0: "auto", 1: "atomic scatter", 2: "inverse-map gather", 3: "column owner"}[args.backward_mode],
-                   "step": "forward kernel + backward kernels (gradient zero-fill folded into the first)"},
+                   "step": "forward kernel + backward kernels (gradient zero-fill folded into the first)",
+                   "submission": "eager launches on one stream"},
+        "ms_per_step_eager": eager_ms, "ms_per_step_graph": graph_ms,
         "fwd_call_ms": stats(fwd), "bwd_call_ms": stats(bwd),
         "effective_GBps_fwd_bwd": (fb + bb) / ms / 1e6,
         "frac_hbm_fwd_bwd": (fb + bb) / ms / 1e6 / HBM_PEAK_GBS,

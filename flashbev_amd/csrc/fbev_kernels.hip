@@ -965,13 +965,16 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
 }
 
 // Texel pass of the inverse-map backward.  A texel's pairs are handled by one block, or, when
-// there are more than kTexelPart of them (the texels on the horizon collect thousands), by up
-// to kTexelSplit blocks (blockIdx.y) that each take an equal share.  A block's
+// the grid has a second dimension and there are more than kTexelPart of them, by up to
+// gridDim.y blocks that each take an equal share.  Every block of a texel first has to read the
+// texel's segment bounds, so idle blocks are not free: the host splits only when there are too
+// few texels to fill the machine otherwise (kTexelSplitBelow).  A block's
 // 4 * (64 / lanes_per_row) workers stride over its pairs, each gathering grad_out rows with
 // 128-bit loads; partial rows meet in LDS.  A texel handled by one block is updated with plain
 // loads and stores; the shares of a split texel are combined with fp32 atomics (at most
-// kTexelSplit per address).
-constexpr int kTexelSplit = 8;
+// gridDim.y per address).
+constexpr int kTexelMaxSplit = 8;
+constexpr int kTexelSplitBelow = 8192;
 constexpr int kTexelPart = 128;
 template <int VEC>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_kernel(
@@ -987,7 +990,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
     int end = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
     if (start >= end) return;      // uniform for the block
     const int n_all = end - start;
-    const int n_parts = min(kTexelSplit, (n_all + kTexelPart - 1) / kTexelPart);
+    const int n_parts = min((int)gridDim.y, (n_all + kTexelPart - 1) / kTexelPart);
     if ((int)blockIdx.y >= n_parts) return;
     {
         const int s0 = start + (int)(((long long)n_all * blockIdx.y) / n_parts);
@@ -1973,12 +1976,14 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const int nw = (kWave / lpr) * kWavesPerBlock;
     const size_t lds = (size_t)nw * (lpr * vec + 2) * sizeof(float);
     const int from_pairs = (d_depth != nullptr && p->depth_distribution != FBEV_CATEGORICAL) ? 1 : 0;
+    long long want_split = kTexelSplitBelow / texels;
+    const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);
     if (vec4)
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels, kTexelSplit), dim3(kWave * kWavesPerBlock), lds,
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels, n_split), dim3(kWave * kWavesPerBlock), lds,
                            st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
     else
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels, kTexelSplit), dim3(kWave * kWavesPerBlock), lds,
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels, n_split), dim3(kWave * kWavesPerBlock), lds,
                            st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
