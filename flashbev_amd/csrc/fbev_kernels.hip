@@ -81,6 +81,11 @@ constexpr int kXcdCount = 8;                 // accelerator complex dies, each w
 // samples, so every texel owns kReplicas counters and a sample picks one from its cell.
 constexpr int kReplicaBits = 5;
 constexpr int kReplicas = 1 << kReplicaBits;
+// With fixed-capacity segments (no counting pass) a texel has one segment per wavefront of the
+// block that later gathers it.
+constexpr int kFixedReplicas = 4;
+constexpr int kFixedMinSegment = 16;          // shorter segments would mostly overflow: count instead
+static_assert(kFixedReplicas == kWavesPerBlock, "one fixed segment per wavefront of the texel block");
 constexpr int kScanChunkBits = 12;           // counters are prefix-summed in chunks of 4096
 
 struct KParams {
@@ -487,21 +492,38 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         if (MODE == kModeFill && keep) {
             // claim one position per corner in the texel's segment of the pair array; the four
             // requests of all lanes are in flight together, so the round trip is paid once
-            const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
-            const int i0 = tx.x * kReplicas + rep, i1 = tx.y * kReplicas + rep;
-            const int i2 = tx.z * kReplicas + rep, i3 = tx.w * kReplicas + rep;
-            int p0 = atomicAdd(cursor + i0, 1);
-            int p1 = atomicAdd(cursor + i1, 1);
-            int p2 = atomicAdd(cursor + i2, 1);
-            int p3 = atomicAdd(cursor + i3, 1);
-            p0 += chunk_prefix[i0 >> kScanChunkBits];
-            p1 += chunk_prefix[i1 >> kScanChunkBits];
-            p2 += chunk_prefix[i2 >> kScanChunkBits];
-            p3 += chunk_prefix[i3 >> kScanChunkBits];
-            p0 = p0 < pair_cap ? p0 : -1;
-            p1 = p1 < pair_cap ? p1 : -1;
-            p2 = p2 < pair_cap ? p2 : -1;
-            p3 = p3 < pair_cap ? p3 : -1;
+            int p0, p1, p2, p3;
+            if (chunk_prefix != nullptr) {
+                // counted segments: cursor holds each segment's start within its scan chunk
+                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
+                const int i0 = tx.x * kReplicas + rep, i1 = tx.y * kReplicas + rep;
+                const int i2 = tx.z * kReplicas + rep, i3 = tx.w * kReplicas + rep;
+                p0 = atomicAdd(cursor + i0, 1);
+                p1 = atomicAdd(cursor + i1, 1);
+                p2 = atomicAdd(cursor + i2, 1);
+                p3 = atomicAdd(cursor + i3, 1);
+                p0 += chunk_prefix[i0 >> kScanChunkBits];
+                p1 += chunk_prefix[i1 >> kScanChunkBits];
+                p2 += chunk_prefix[i2 >> kScanChunkBits];
+                p3 += chunk_prefix[i3 >> kScanChunkBits];
+                p0 = p0 < pair_cap ? p0 : -1;
+                p1 = p1 < pair_cap ? p1 : -1;
+                p2 = p2 < pair_cap ? p2 : -1;
+                p3 = p3 < pair_cap ? p3 : -1;
+            } else {
+                // fixed segments of pair_cap pairs per (texel, replica): cursor counts from zero
+                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16) & (kFixedReplicas - 1);
+                const int i0 = tx.x * kFixedReplicas + rep, i1 = tx.y * kFixedReplicas + rep;
+                const int i2 = tx.z * kFixedReplicas + rep, i3 = tx.w * kFixedReplicas + rep;
+                p0 = atomicAdd(cursor + i0, 1);
+                p1 = atomicAdd(cursor + i1, 1);
+                p2 = atomicAdd(cursor + i2, 1);
+                p3 = atomicAdd(cursor + i3, 1);
+                p0 = p0 < pair_cap ? i0 * pair_cap + p0 : -1;
+                p1 = p1 < pair_cap ? i1 * pair_cap + p1 : -1;
+                p2 = p2 < pair_cap ? i2 * pair_cap + p2 : -1;
+                p3 = p3 < pair_cap ? i3 * pair_cap + p3 : -1;
+            }
             float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
             e[ENTRY_F4 - 1] = make_float4(__int_as_float(p0), __int_as_float(p1), __int_as_float(p2),
                                           __int_as_float(p3));
@@ -984,24 +1006,39 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
     extern __shared__ float4 smem[];
     float *part = reinterpret_cast<float *>(smem);
     const int t = blockIdx.x;
-    // the texel's pairs: from the end of the previous texel's last replica to the end of its own
-    const long long first = (long long)t * kReplicas - 1, last = (long long)t * kReplicas + kReplicas - 1;
-    int start = t == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
-    int end = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
-    if (start >= end) return;      // uniform for the block
-    const int n_all = end - start;
-    const int n_parts = min((int)gridDim.y, (n_all + kTexelPart - 1) / kTexelPart);
-    if ((int)blockIdx.y >= n_parts) return;
-    {
-        const int s0 = start + (int)(((long long)n_all * blockIdx.y) / n_parts);
-        const int s1 = start + (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
-        start = s0;
-        end = s1;
-    }
-    const bool shared_texel = n_parts > 1;
-    const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
+    // this wavefront's pairs: [wave_start, wave_end) in steps of wave_stride
+    int wave_start, wave_end, wave_stride;
+    bool shared_texel;
+    if (chunk_prefix != nullptr) {
+        // counted segments, one after the other: from the end of the previous texel's last
+        // replica to the end of this texel's; the wavefronts interleave
+        const long long first = (long long)t * kReplicas - 1, last = (long long)t * kReplicas + kReplicas - 1;
+        int start = t == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
+        int end = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
+        if (start >= end) return;      // uniform for the block
+        const int n_all = end - start;
+        const int n_parts = min((int)gridDim.y, (n_all + kTexelPart - 1) / kTexelPart);
+        if ((int)blockIdx.y >= n_parts) return;
+        wave_start = start + (int)(((long long)n_all * blockIdx.y) / n_parts) + wave * kWave;
+        wave_end = start + (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
+        wave_stride = kWavesPerBlock * kWave;
+        shared_texel = n_parts > 1;
+    } else {
+        // fixed segments of pair_cap pairs, one per wavefront; seg_end holds how many were claimed
+        const int4 c = *reinterpret_cast<const int4 *>(seg_end + (size_t)t * kFixedReplicas);
+        const int n_max = min(max(max(c.x, c.y), max(c.z, c.w)), pair_cap);
+        const int n_parts = min((int)gridDim.y, (n_max + kTexelPart - 1) / kTexelPart);
+        if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
+        const int mine = min(wave == 0 ? c.x : (wave == 1 ? c.y : (wave == 2 ? c.z : c.w)), pair_cap);
+        const int base = (t * kFixedReplicas + wave) * pair_cap;
+        wave_start = base + (int)(((long long)mine * blockIdx.y) / n_parts);
+        wave_end = base + (int)(((long long)mine * (blockIdx.y + 1)) / n_parts);
+        wave_stride = kWave;
+        shared_texel = n_parts > 1;
+    }
+    const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
     const int wpw = kWave / lanes_per_row;            // workers per wavefront
     const int nw = wpw * kWavesPerBlock;
     const int wslot = lane / lanes_per_row;
@@ -1021,8 +1058,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
         // load, and hands them to its workers through lane shuffles; four grad_out rows per
         // worker are in flight before the first is used.  The loop is bound by load latency:
         // without this the pair load and the row load it addresses form a dependent chain.
-        for (int bstart = start + wave * kWave; bstart < end; bstart += kWavesPerBlock * kWave) {
-            const int nb = min(kWave, end - bstart);
+        for (int bstart = wave_start; bstart < wave_end; bstart += wave_stride) {
+            const int nb = min(kWave, wave_end - bstart);
             float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f);
             if (lane < nb) pr = *reinterpret_cast<const float4 *>(pairs + bstart + lane);
             // a pair is written by the cell pass before this kernel starts; the range check
@@ -1944,27 +1981,37 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const long long counters = counter_count(p), chunks = chunk_count(p);
     int *chunk_prefix = cursor + counters;
 
-    rc = launch_zero(cursor, counters, accumulate ? nullptr : d_depth, texels * p->depth_bins,
-                     accumulate ? nullptr : d_feats, texels * p->channels, st);
+    // A workspace with room for every sample corner gets fixed segments: each (texel, replica)
+    // owns cap / (texels * kFixedReplicas) pair slots, and the counting pass and the prefix sums
+    // are not needed.  (A texel that outgrows its segments falls back to atomics, like a full
+    // pair array does.)  Smaller workspaces are packed exactly: count, scan, fill.
+    const bool fixed = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (texels * kFixedReplicas) >= kFixedMinSegment;
+    const int seg_cap = fixed ? (int)(cap / (texels * kFixedReplicas)) : 0;
+    rc = launch_zero(cursor, fixed ? texels * kFixedReplicas : counters, accumulate ? nullptr : d_depth,
+                     texels * p->depth_bins, accumulate ? nullptr : d_feats, texels * p->channels, st);
     if (rc != FBEV_OK) return rc;
-    switch (p->in_dtype) {
-        case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, st); break;
-        case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, st); break;
-        default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, st); break;
+    if (!fixed) {
+        switch (p->in_dtype) {
+            case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, st); break;
+            case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, st); break;
+            default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, st); break;
+        }
+        if (rc != FBEV_OK) return rc;
+        {
+            prof::Scope timer(prof::kScanChunks, st);
+            hipLaunchKernelGGL(fbev_scan_chunks_kernel, dim3((unsigned)chunks), dim3(1024), 0, st, cursor, counters,
+                               chunk_prefix);
+        }
+        if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+        {
+            prof::Scope timer(prof::kScanSums, st);
+            hipLaunchKernelGGL(fbev_scan_sums_kernel, dim3(1), dim3(1024), 0, st, chunk_prefix, (int)chunks);
+        }
+        if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
     }
-    if (rc != FBEV_OK) return rc;
-    {
-        prof::Scope timer(prof::kScanChunks, st);
-        hipLaunchKernelGGL(fbev_scan_chunks_kernel, dim3((unsigned)chunks), dim3(1024), 0, st, cursor, counters,
-                           chunk_prefix);
-    }
-    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
-    {
-        prof::Scope timer(prof::kScanSums, st);
-        hipLaunchKernelGGL(fbev_scan_sums_kernel, dim3(1), dim3(1024), 0, st, chunk_prefix, (int)chunks);
-    }
-    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
-    rc = dispatch_cells<true>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, chunk_prefix, cursor, pairs, cap,
+    const int *prefix_arg = fixed ? nullptr : chunk_prefix;
+    const int cap_arg = fixed ? seg_cap : cap;
+    rc = dispatch_cells<true>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs, cap_arg,
                               st);
     if (rc != FBEV_OK) return rc;
 
@@ -1981,10 +2028,10 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     prof::Scope timer(prof::kBackwardTexel, st);
     if (vec4)
         hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels, n_split), dim3(kWave * kWavesPerBlock), lds,
-                           st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
+                           st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
     else
         hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels, n_split), dim3(kWave * kWavesPerBlock), lds,
-                           st, pl.k, grad_out, chunk_prefix, cursor, pairs, cap, d_depth, d_feats, lpr, from_pairs);
+                           st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 

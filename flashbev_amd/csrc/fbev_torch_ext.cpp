@@ -234,11 +234,12 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                                      ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, st);
     };
     // Inverse-map gather.  The pair array comes from PyTorch's caching allocator (no device
-    // allocation in steady state).  Half of the worst case holds every rig whose cameras see
-    // less than half of all (cell, height) samples; what does not fit is applied with atomics.
+    // allocation in steady state).  By default it has room for every sample corner, which lets
+    // the library use fixed per-texel segments and skip its counting pass; a smaller
+    // pair_capacity selects the exactly packed layout (what does not fit is applied with atomics).
     auto run_gather = [&]() -> int {
         const uint64_t max_pairs = fbev_backward_max_pairs(&p);
-        uint64_t cap = pair_capacity >= 0 ? (uint64_t)pair_capacity : (max_pairs + 1) / 2;
+        uint64_t cap = pair_capacity >= 0 ? (uint64_t)pair_capacity : max_pairs;
         if (cap > max_pairs) cap = max_pairs;
         const size_t bytes = fbev_backward_workspace_bytes(&p, cap);
         at::Tensor ws = at::empty({(int64_t)bytes}, at::TensorOptions().device(depth_params.device()).dtype(at::kByte));

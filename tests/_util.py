@@ -79,12 +79,13 @@ def capi_forward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN
 def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, want=(True, True),
                   mode="scatter", pair_capacity=None):
     """Backward through the C ABI.  mode "scatter" = fbev_backward, "gather" = fbev_backward_gather
-    with a workspace for `pair_capacity` pairs (default: the worst case), "columns" =
+    with a workspace for `pair_capacity` pairs (default: the worst case, which selects fixed
+    per-texel segments; "gather_counted" defaults to half of that, the exactly packed layout), "columns" =
     fbev_backward_columns overwriting NaN-filled buffers with recounted cell counts,
     "columns_acc" = the same accumulating into zero-filled buffers with the forward's counts."""
     p = problem_for(x, w, dist, thr, eps, reduction)
     dev = x["image_feats"].device
-    overwrite = mode in ("columns", "scatter_overwrite", "gather_overwrite")
+    overwrite = mode in ("columns", "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite")
     fill = float("nan") if overwrite else 0.0
     dd = torch.full(x["depth_params"].shape, fill, dtype=torch.float32, device=dev) if want[0] else None
     df = torch.full(x["image_feats"].shape, fill, dtype=torch.float32, device=dev) if want[1] else None
@@ -108,7 +109,9 @@ def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEA
             capi.check(capi.backward_columns(p, *args, cnt.data_ptr(), ddp, dfp, True, None, 0, st),
                        "fbev_backward_columns")
     else:
-        cap = capi.backward_max_pairs(p) if pair_capacity is None else pair_capacity
+        cap = pair_capacity
+        if cap is None:
+            cap = capi.backward_max_pairs(p) // (2 if mode.startswith("gather_counted") else 1)
         nbytes = capi.backward_workspace_bytes(p, cap)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         capi.check(capi.backward_gather(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),

@@ -56,8 +56,8 @@ def test_forward_matches_c_oracle(name, dist, thr):
 
 @pytest.mark.parametrize("name", ["cfg1_tiny", "cfg2_surround"])
 @pytest.mark.parametrize("dist", [0, 1, 2])
-@pytest.mark.parametrize("mode", ["scatter", "gather", "columns", "columns_acc", "scatter_overwrite",
-                                  "gather_overwrite"])
+@pytest.mark.parametrize("mode", ["scatter", "gather", "gather_counted", "columns", "columns_acc",
+                                  "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite"])
 def test_backward_matches_c_oracle(name, dist, mode):
     w, x = _inputs(name, dist)
     dd, df = U.capi_backward(x, w, dist, mode=mode)
@@ -81,7 +81,7 @@ def test_backward_single_gradient():
     """Either gradient pointer may be NULL."""
     w, x = _inputs("cfg2_surround", 0)
     want_dd, want_df = U.oracle_backward(x, w, 0)
-    for mode in ("scatter", "gather", "columns"):
+    for mode in ("scatter", "gather", "gather_counted", "columns"):
         dd, df = U.capi_backward(x, w, 0, mode=mode, want=(True, False))
         assert df is None and U.violations(dd.cpu().numpy(), want_dd)[0] == 0
         dd, df = U.capi_backward(x, w, 0, mode=mode, want=(False, True))

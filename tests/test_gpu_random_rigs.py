@@ -68,7 +68,7 @@ def test_random_rig(seed):
     bad, maxabs, ratio = U.violations(out.cpu().numpy(), want)
     assert bad == 0, (bad, maxabs, ratio)
     want_dd, want_df = U.oracle_backward(x, w, dist, thr)
-    for mode in ("scatter", "gather", "columns", "columns_acc", "gather_overwrite"):
+    for mode in ("scatter", "gather", "gather_counted", "columns", "columns_acc", "gather_overwrite"):
         dd, df = U.capi_backward(x, w, dist, thr, mode=mode)
         for got, r, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
             bad, maxabs, ratio = U.violations(got.cpu().numpy(), r)

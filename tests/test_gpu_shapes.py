@@ -22,7 +22,7 @@ def small(name="cfg2_surround", **kw):
     return dataclasses.replace(WORKLOADS[name], **kw)
 
 
-def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "columns"), fwd_tol=(1e-4, 1e-5)):
+def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "gather_counted", "columns"), fwd_tol=(1e-4, 1e-5)):
     out = U.capi_forward(x, w, dist, thr).cpu().numpy()
     want = U.oracle_forward(x, w, dist, thr)
     bad, maxabs, ratio = U.violations(out, want, *fwd_tol)
@@ -54,7 +54,8 @@ def test_channel_counts_off_the_vector_path(channels):
     check_all(w, x, 1)
 
 
-@pytest.mark.parametrize("channels,dtype", [(512, torch.float32), (1024, torch.float32), (2048, torch.float16)])
+@pytest.mark.parametrize("channels,dtype", [(512, torch.float32), (1024, torch.float32), (1028, torch.float32),
+                                            (2048, torch.float16)])
 def test_wide_channels(channels, dtype):
     w = small("cfg1_tiny", channels=channels, dtype=dtype, grid_size=(16, 16, 3))
     x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
@@ -103,7 +104,7 @@ def test_sum_reduction(dist):
     want = U.oracle_forward(x, w, dist, reduce_sum=True)
     assert U.violations(out, want)[0] == 0
     want_dd, want_df = U.oracle_backward(x, w, dist, reduce_sum=True)
-    for mode in ("scatter", "gather", "columns"):
+    for mode in ("scatter", "gather", "gather_counted", "columns"):
         dd, df = U.capi_backward(x, w, dist, reduction=capi.FBEV_REDUCE_SUM, mode=mode)
         assert U.violations(df.cpu().numpy(), want_df)[0] == 0
         assert U.violations(dd.cpu().numpy(), want_dd)[0] == 0
@@ -191,8 +192,9 @@ def test_full_size_properties(name, dist):
     two = dict(x, image_feats=(x["image_feats"] * 2).contiguous())
     assert torch.equal(U.capi_forward(two, w, dist), out * 2)
     dd, df = U.capi_backward(x, w, dist, mode="columns")
-    ddg, dfg = U.capi_backward(x, w, dist, mode="gather")
-    assert torch.allclose(df, dfg, rtol=1e-4, atol=1e-5) and torch.allclose(dd, ddg, rtol=1e-3, atol=1e-4)
+    for gather_mode in ("gather", "gather_counted"):
+        ddg, dfg = U.capi_backward(x, w, dist, mode=gather_mode)
+        assert torch.allclose(df, dfg, rtol=1e-4, atol=1e-5) and torch.allclose(dd, ddg, rtol=1e-3, atol=1e-4)
     lhs = (out.double() * x["grad_out"].double()).sum().item()
     rhs = (df.double() * x["image_feats"].double()).sum().item()
     assert abs(lhs - rhs) <= 2e-4 * max(abs(lhs), abs(rhs), 1.0), (lhs, rhs)
