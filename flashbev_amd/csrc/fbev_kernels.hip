@@ -297,10 +297,16 @@ __device__ __forceinline__ unsigned long long lanemask_le(int lane) { return ~0u
 //   [matrices: N*12 floats][decode table: slots*NZ ints]
 //   per wavefront: [16 ints of list lengths][16 float4 of cell centres][slots*NZ ints of
 //   candidates][slots * list_cap entries]
+// Counters that several lanes of a wavefront update in turn live in LDS and are read as
+// volatile.  The pointer carries the LDS address space: a volatile access through a generic
+// pointer becomes a system-coherent flat load that first waits for every outstanding global
+// store and atomic of the wavefront.
+using lds_counter = volatile __attribute__((address_space(3))) int;
+
 struct WaveLds {
     const float *Pm;
     const int *dec;       // sample index within the wavefront's round -> slot << 28 | camera << 16 | height bin
-    volatile int *cnt;    // entries per slot
+    lds_counter *cnt;     // entries per slot
     float4 *cell;         // per slot: x, y, valid flag, ix | iy << 16
     int *cand;            // samples that survive the cheap test
     float4 *lst;
@@ -321,7 +327,7 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
     float4 *wbase = smem + lds_p_f4(k) + dec_f4 + (threadIdx.x >> 6) * per_wave_f4;
     L.Pm = Pm;
     L.dec = dec;
-    L.cnt = reinterpret_cast<volatile int *>(wbase);
+    L.cnt = (lds_counter *)reinterpret_cast<int *>(wbase);
     L.cell = wbase + 4;
     L.cand = reinterpret_cast<int *>(wbase + 20);
     L.lst = wbase + 20 + dec_f4;
@@ -545,7 +551,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     const int blk = bid - b * k.blocks_per_batch;
 
     const WaveLds L = block_lds_setup(k, smem, proj, b, 2);
-    volatile int *cnt = L.cnt;
+    lds_counter *cnt = L.cnt;
     float4 *lst = L.lst;
 
     const int cells_per_wave = k.slots * k.rounds;
@@ -769,7 +775,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     const int blk = bid - b * k.blocks_per_batch;
 
     const WaveLds L = block_lds_setup(k, smem, proj, b, EF4);
-    volatile int *cnt = L.cnt;
+    lds_counter *cnt = L.cnt;
     float4 *lst = L.lst;
 
     const int cells_per_wave = k.slots * k.rounds;
@@ -1172,17 +1178,18 @@ struct ColParams {
 
 struct ColLds {
     float *Pm;
-    volatile int *ctrl;    // 0: tiles kept, 1: cells kept, 2: entries
+    lds_counter *ctrl;     // 0: tiles kept, 1: cells kept, 2: entries
     int *tiles, *cells, *contrib, *rowcnt, *rowstart, *rowfill, *wk_row, *wk_first, *wk_n;
     float4 *entries;
     float *G, *part;
 };
 
 // Append `keep` lanes' values to a list with one LDS atomic per wavefront.
-__device__ __forceinline__ int wave_append(volatile int *counter, bool keep, int lane) {
+__device__ __forceinline__ int wave_append(lds_counter *counter, bool keep, int lane) {
     const unsigned long long m = __ballot(keep);
     int base = 0;
-    if (lane == 0 && m != 0ull) base = atomicAdd(const_cast<int *>(counter), __popcll(m));
+    if (lane == 0 && m != 0ull) base = __hip_atomic_fetch_add((__attribute__((address_space(3))) int *)counter, __popcll(m), __ATOMIC_RELAXED,
+                                                                __HIP_MEMORY_SCOPE_WORKGROUP);
     base = __shfl(base, 0, kWave);
     return base + __popcll(m & lanemask_lt(lane));
 }
@@ -1419,7 +1426,7 @@ __global__ __launch_bounds__(kColThreads) void fbev_backward_column_kernel(
     const int n_workers = kColWaves * cp.slots;
     ColLds L;
     L.Pm = reinterpret_cast<float *>(smem);
-    L.ctrl = reinterpret_cast<volatile int *>(smem + 4);
+    L.ctrl = (lds_counter *)reinterpret_cast<int *>(smem + 4);
     L.entries = smem + 8;
     int *ip = reinterpret_cast<int *>(L.entries + 2 * kColEntries);
     L.tiles = ip; ip += kColThreads;
