@@ -107,6 +107,7 @@ struct KParams {
     int reduce_sum;
     int proj_stride;
     int n_blocks;
+    int bin_bits;        // a pair's first word is cell << bin_bits | depth bin; -1: the word cannot hold both
 };
 
 // ---------------------------------------------------------------- element access
@@ -791,6 +792,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     // G of four entries is summed over the lanes of a slot at a time when the slots start on
     // multiples of four lanes (always, on the 128-bit path)
     const bool grouped = (k.lanes_per_slot & 3) == 0;
+    // The depth gradient travels with the pairs when one channel pass sees the whole of G and
+    // the pair's first word has room for the depth bin; otherwise it is added with atomics here.
+    const bool fold = FILL && need_G && k.C <= span && k.bin_bits >= 0;
 
     for (int r = 0; r < k.rounds; ++r) {
         const int q0 = (blk * kWavesPerBlock + wave) * cells_per_wave + r * k.slots;
@@ -894,13 +898,13 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
             };
             // what one lane does with the complete G of entry e
             auto entry_done = [&](int e, float G) {
-                if (FILL && first_pass && parametric) {
-                    // the pairs are written after the loop, 64 at a time; keep G with the entry
-                    // (the bin word of a parametric entry is unused)
-                    my[EF4 * e + 1].w = G;
+                if (fold) {
+                    // the pairs are written after the loop, 64 at a time; keep G * (a, b) with the
+                    // entry in place of (a, b)
+                    my[EF4 * e + 1].y *= G;
+                    my[EF4 * e + 1].z *= G;
                 } else {
-                    // scatter path, categorical bins, or a later channel pass whose share of G
-                    // cannot be folded into a pair already written
+                    // scatter path, or G arrives in several channel passes
                     const float4 geo = my[EF4 * e], dw = my[EF4 * e + 1];
                     const float du = geo.x, dv = geo.y;
                     const float wc[4] = {(1.0f - du) * (1.0f - dv), (1.0f - du) * dv, du * (1.0f - dv), du * dv};
@@ -973,16 +977,19 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                         const float wu = (c & 2) ? du : 1.0f - du, wv = (c & 1) ? dv : 1.0f - dv;
                         const float wcc = wu * wv;
                         const int posc = __float_as_int(c == 0 ? pfp.x : (c == 1 ? pfp.y : (c == 2 ? pfp.z : pfp.w)));
-                        const float Gp = (need_G && parametric) ? dwp.w : 0.0f;   // already carries 1/count
-                        const float da = Gp * dwp.y * wcc, db = Gp * dwp.z * wcc;
+                        // G * a and G * b (G already carries 1/count)
+                        const float da = fold ? dwp.y * wcc : 0.0f, db = fold ? dwp.z * wcc : 0.0f;
+                        const int kk = __float_as_int(dwp.w);
+                        const int k0 = parametric ? 0 : (kk & 0xffff), k1 = parametric ? 1 : (kk >> 16);
                         if (posc >= 0) {
+                            const int word = fold ? ((pcell << k.bin_bits) | k0) : pcell;
                             *reinterpret_cast<float4 *>(pairs + posc) =
-                                make_float4(__int_as_float(pcell), wcc * dwp.x * pinv, da, db);
-                        } else if (need_G && parametric) {
+                                make_float4(__int_as_float(word), wcc * dwp.x * pinv, da, db);
+                        } else if (fold) {
                             const int fl = __float_as_int(geo.w);
                             const int tt = __float_as_int(geo.z) + ((c & 1) && (fl & 2) ? k.W : 0) + ((c & 2) ? (fl & 1) : 0);
-                            atomic_add_f32(d_depth + (size_t)tt * 2, da);
-                            atomic_add_f32(d_depth + (size_t)tt * 2 + 1, db);
+                            atomic_add_f32(d_depth + (size_t)tt * Dd + k0, da);
+                            atomic_add_f32(d_depth + (size_t)tt * Dd + k1, db);
                         }
                     }
                 }
@@ -1053,6 +1060,14 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
     const int worker = wave * wpw + wslot;
     const int span = lanes_per_row * VEC;
     const int stride = span + 2;                      // partial row + the two depth sums
+    // categorical depth gradient: one LDS accumulator per depth bin of this texel
+    const bool bin_sums = depth_from_pairs && k.dist == FBEV_CATEGORICAL;
+    float *bins = part + nw * stride;
+    const int bin_bits = depth_from_pairs ? k.bin_bits : 0, bin_mask = (1 << bin_bits) - 1;
+    if (bin_sums) {
+        for (int i = threadIdx.x; i < k.Dd; i += blockDim.x) bins[i] = 0.0f;
+        __syncthreads();
+    }
     for (int c0 = 0; c0 < k.C; c0 += span) {
         const int ch = c0 + lir * VEC;
         const bool on = worker_lane && ch < k.C;
@@ -1070,10 +1085,20 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
             if (lane < nb) pr = *reinterpret_cast<const float4 *>(pairs + bstart + lane);
             // a pair is written by the cell pass before this kernel starts; the range check
             // only keeps a logic error from turning into a wild read
-            const bool valid = (unsigned)__float_as_int(pr.x) < n_cells;
-            const int my_cell = valid ? __float_as_int(pr.x) : -1;
+            const int word = __float_as_int(pr.x);
+            const bool valid = (unsigned)(word >> bin_bits) < n_cells;
+            const int my_cell = valid ? (word >> bin_bits) : -1;
             const float my_coef = valid ? pr.y : 0.0f;
-            if (c0 == 0 && valid) { sa += pr.z; sb += pr.w; }
+            if (c0 == 0 && valid) {
+                if (bin_sums) {
+                    const int k0 = word & bin_mask;
+                    __hip_atomic_fetch_add(bins + k0, pr.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(bins + min(k0 + 1, k.Dd - 1), pr.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                } else {
+                    sa += pr.z;
+                    sb += pr.w;
+                }
+            }
             constexpr int UNR = 4;
             for (int i = 0; i < nb; i += wpw * UNR) {
                 int cells[UNR];
@@ -1129,7 +1154,16 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
                 else *dst += sum;
             }
         }
-        if (c0 == 0 && depth_from_pairs && threadIdx.x < 2) {
+        if (c0 == 0 && bin_sums) {
+            for (int i = threadIdx.x; i < k.Dd; i += blockDim.x) {
+                const float sum = bins[i];
+                if (sum != 0.0f) {
+                    float *dst = d_depth + (size_t)t * k.Dd + i;
+                    if (shared_texel) atomic_add_f32(dst, sum);
+                    else *dst += sum;
+                }
+            }
+        } else if (c0 == 0 && depth_from_pairs && threadIdx.x < 2) {
             float sum = 0.0f;
             for (int w = 0; w < nw; ++w) sum += part[w * stride + span + threadIdx.x];
             float *dst = d_depth + (size_t)t * 2 + threadIdx.x;
@@ -1684,6 +1718,12 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan) {
     k.dmin = p->depth_min; k.dstep = p->depth_step;
     k.reduce_sum = p->reduction == FBEV_REDUCE_SUM;
     k.proj_stride = p->proj_stride;
+    {
+        int bits = 0;
+        if (k.dist == FBEV_CATEGORICAL) while ((1 << bits) < k.Dd) ++bits;
+        const long long cells = (long long)k.B * p->grid_y * p->grid_x;
+        k.bin_bits = (cells << bits) < (1ll << 31) ? bits : -1;
+    }
 
     const int es = elem_size(p->in_dtype);
     const int full_vec = 16 / es;
@@ -2028,8 +2068,12 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const int cq = (p->channels + vec - 1) / vec;
     const int lpr = cq < kWave ? cq : kWave;
     const int nw = (kWave / lpr) * kWavesPerBlock;
-    const size_t lds = (size_t)nw * (lpr * vec + 2) * sizeof(float);
-    const int from_pairs = (d_depth != nullptr && p->depth_distribution != FBEV_CATEGORICAL) ? 1 : 0;
+    // the depth gradient rides on the pairs exactly when the cell pass folds it in (one channel pass
+    // and room for the depth bin in a pair's first word)
+    const int from_pairs =
+        (d_depth != nullptr && pl.k.C <= pl.k.lanes_per_slot * pl.vec * pl.cpl && pl.k.bin_bits >= 0) ? 1 : 0;
+    const size_t lds = ((size_t)nw * (lpr * vec + 2) + (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) *
+                       sizeof(float);
     long long want_split = kTexelSplitBelow / texels;
     const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);
