@@ -7,6 +7,12 @@ gets +0.1), the calibration tensors of the BEVDet-style input list become 3x4 pr
 matrices, and ``flash_bevpool`` pools them into ``[B, C, Y, X]``.  Parameter and buffer names
 match the reference, so its state dicts load.
 
+The two 1x1 convolutions are applied as matrix products that write channels-last results
+directly, so the channels-last copy of the feature and depth maps that the reference makes on
+every call (sampling_vt.py:252-253, flash_bevpool.py:47-48) does not exist here, whatever the
+memory format of the incoming feature map; the ``[B, C, Y, X]`` result is a view of the
+operator's ``[B, Y, X, C]`` output (channels-last memory format), not a copy.
+
 Only the fused path exists here: ``fuse_projection=False`` (the reference's dense PyTorch and
 PillarPool branches, sampling_vt.py:269-292) raises.  Grid sizes are rounded, not truncated
 (the reference's float-to-int32 truncation at sampling_vt.py:189-193 can lose a cell when
@@ -16,6 +22,7 @@ from __future__ import annotations
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from .flash_bevpool import flash_bevpool
 from .rig import create_projection_matrix
@@ -59,27 +66,44 @@ class SamplingVT(nn.Module):
         self._roi_host = [float(v) for a in axes for v in a[:2]]
         self._grid_host = sizes
 
+    @staticmethod
+    def _pointwise(conv, x):
+        """A 1x1 convolution of ``x [M, C, H, W]`` with channels-last output ``[M, H, W, C_out]``:
+        a matrix product over a transposed view of ``x`` (no copy for either memory format)."""
+        M, C, H, W = x.shape
+        rows = x.permute(0, 2, 3, 1).reshape(M, H * W, C) if x.is_contiguous(memory_format=torch.channels_last) \
+            else x.flatten(2).transpose(1, 2)
+        return F.linear(rows, conv.weight.flatten(1), conv.bias).unflatten(1, (H, W))
+
+    def _depth_last(self, x):
+        d = torch.relu(self._pointwise(self.depth_network[0], x))
+        return torch.stack([d[..., 0], d[..., 1] + 0.1], dim=-1)
+
     def forward_depth(self, x):
-        depth_params = self.depth_network(x)
-        mean, sigma = depth_params[:, 0:1], depth_params[:, 1:2] + 0.1
-        return torch.cat([mean, sigma], dim=1)
+        """Per-pixel (mean, sigma) as ``[M, 2, H, W]`` (sigma gets +0.1), like the reference."""
+        return self._depth_last(x).movedim(-1, 1)
 
     def forward(self, input, images=None, img_meta=None, lidar_cloud=None, depth_from_lidar=None):
         x = input[0]
         B, N, C, H, W = x.shape
         x = x.reshape(B * N, C, H, W)
-        features_pv = self.context_network(x)
-        depths = self.forward_depth(x)
-        return self.sampling_vt(input, features_pv, depths), depths
+        features_last = self._pointwise(self.context_network, x)     # [B*N, H, W, C_out]
+        depths_last = self._depth_last(x)                            # [B*N, H, W, 2]
+        bev = self._pool(input, features_last, depths_last)
+        return bev, depths_last.movedim(-1, 1)
 
     def sampling_vt(self, input, features_pv, depths):
+        """Reference entry point with channels-first maps ``[B*N, C, H, W]`` / ``[B*N, 2, H, W]``."""
+        return self._pool(input, features_pv.movedim(-3, -1), depths.movedim(-3, -1))
+
+    def _pool(self, input, features_last, depths_last):
         B, N = input[3].shape[:2]
         projection_matrices = create_projection_matrix(*input[1:7])
-        H, W = features_pv.shape[-2:]
+        H, W = features_last.shape[1:3]
         feature_size = torch.tensor([H, W], dtype=torch.int32).repeat(B, N, 1)
         bev_feat = flash_bevpool(
-            image_feats=features_pv.movedim(-3, -1).unflatten(0, (B, N)),
-            depth_params=depths.movedim(-3, -1).unflatten(0, (B, N)),
+            image_feats=features_last.unflatten(0, (B, N)),
+            depth_params=depths_last.unflatten(0, (B, N)),
             projection_matrices=projection_matrices,
             feature_size=feature_size,
             image_size=list(self.image_size),

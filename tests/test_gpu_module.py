@@ -44,6 +44,24 @@ def test_module_state_dict_names_and_buffers():
     assert SamplingVT(g2, (256, 704), in_channels=8, out_channels=4).sample_grid_size.tolist()[2] == 12
 
 
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_pointwise_heads_equal_the_convolutions_and_write_channels_last(channels_last):
+    """The module applies its 1x1 convolutions as matrix products whose output is already
+    channels-last; the values are those of nn.Conv2d with the same parameters."""
+    torch.manual_seed(3)
+    vt = SamplingVT(GRID, (256, 704), in_channels=32, out_channels=24)
+    x = torch.randn(6, 32, 16, 44)
+    if channels_last:
+        x = x.contiguous(memory_format=torch.channels_last)
+    f = vt._pointwise(vt.context_network, x)
+    assert f.shape == (6, 16, 44, 24) and f.is_contiguous()
+    assert torch.allclose(f, vt.context_network(x).movedim(1, -1), rtol=1e-5, atol=1e-5)
+    d = vt.forward_depth(x)
+    want = vt.depth_network(x)
+    want = torch.cat([want[:, 0:1], want[:, 1:2] + 0.1], dim=1)
+    assert d.shape == want.shape and torch.allclose(d, want, rtol=1e-5, atol=1e-5)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("depth_distribution", ["laplace", "gaussian"])
 def test_module_matches_dense_path(depth_distribution):
@@ -51,6 +69,7 @@ def test_module_matches_dense_path(depth_distribution):
     with torch.no_grad():
         bev, depths = vt(inp)
     assert bev.shape == (1, 24, 100, 100) and depths.shape == (6, 2, 16, 44)
+    assert bev.is_contiguous(memory_format=torch.channels_last)      # a view of [B, Y, X, C], no copy
     # dense path on the CPU with the module's own convolution outputs
     cpu = vt.to("cpu")
     x = inp[0].cpu().reshape(6, -1, 16, 44)

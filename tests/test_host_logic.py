@@ -240,3 +240,24 @@ def test_product_never_imports_the_oracle():
             if fn.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, fn)).read()
                 assert "oracle" not in text.replace("oracle-free", ""), f"{fn} mentions the oracle"
+
+
+def test_latency_sweep_harness_selects_experiments_and_keeps_the_reference_schema():
+    """flashbev_amd.profile_latency mirrors tools/profile_latency.py: one swept list, the
+    reference's record keys and statistics."""
+    from flashbev_amd import profile_latency as pl
+
+    args = pl.parse_args(["--num-cameras-list", "1", "3", "6"])
+    exp = pl.experiment_of(args)
+    assert exp == {"experiment_type": "cameras", "values": [1, 3, 6], "default_bins": 12}
+    assert pl.experiment_of(pl.parse_args([]))["values"] == [12]
+    assert pl.experiment_of(pl.parse_args(["--depth-weight-threshold-list", "0", "1e-4"]))["experiment_type"] == \
+        "depth_threshold"
+    with pytest.raises(ValueError):
+        pl.experiment_of(pl.parse_args(["--num-height-bins", "8", "--num-cameras-list", "2"]))
+    grid = pl.grid_for(args, 20)
+    assert grid["z"] == [-4.0, 2.0, 0.3] and grid["x"] == [-50.0, 50.0, 0.25]
+    stats = pl.latency_stats([1.0, 2.0, 3.0, 4.0])
+    assert set(stats) == {"latency_mean_ms", "latency_std_ms", "latency_min_ms", "latency_max_ms", "latency_p50_ms",
+                          "latency_p95_ms", "latency_p99_ms"}
+    assert stats["latency_mean_ms"] == 2.5 and stats["latency_p50_ms"] == 2.5
