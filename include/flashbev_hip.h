@@ -101,14 +101,18 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
 
 /*
  * Backward through an inverse map (texel -> contributing samples): the same gradients as
- * fbev_backward, formed without floating-point atomics on the feature gradient.  The call
- * counts the contributing sample corners per texel, prefix-sums the counts, writes one
- * 16-byte (cell, coefficient) pair per corner into the texel's segment of the workspace and
- * then gathers per texel.  `accumulate` as in fbev_backward.  `workspace` is caller-owned device memory, 16-byte aligned, of at least
- * fbev_backward_workspace_bytes(p, 0) bytes; pairs that do not fit its capacity are applied
- * with atomics instead, so any capacity gives correct results and
- * fbev_backward_workspace_bytes(p, fbev_backward_max_pairs(p)) never overflows.  The
- * workspace carries no state between calls.
+ * fbev_backward, formed without floating-point atomics on the feature gradient.  The cell
+ * pass writes one 16-byte (cell, coefficient) pair per sample corner into the texel's segment
+ * of the workspace, the texel pass gathers per texel.  `accumulate` as in fbev_backward.
+ * `workspace` is caller-owned device memory, 16-byte aligned, of at least
+ * fbev_backward_workspace_bytes(p, 0) bytes, and carries no state between calls.  Its pair
+ * capacity selects the layout:
+ *   - room for fbev_backward_max_pairs(p) pairs or more: every texel owns fixed segments
+ *     (capacity / texels pair slots, in four replicas) and the call is three launches;
+ *   - anything smaller: the call first counts the sample corners per texel and prefix-sums
+ *     the counts, so that the pairs are packed exactly (two more passes over the samples).
+ * Pairs that find no room (a full segment, or a packed array shorter than the number of
+ * pairs) are applied with atomics instead, so any capacity gives correct results.
  * It is the deterministic-gather alternative to the atomic scatter of
  * flash_bevpool_grad_kernel (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:570-681); the sorted
  * (cell -> sample) intervals of flashbev/flashbevpool/sampling_vt.py:296-311 are the same idea
