@@ -214,3 +214,21 @@ def test_full_size_against_oracle_on_one_batch_element():
     want = U.oracle_forward(one, w1, 1)
     bad, maxabs, ratio = U.violations(out[:1].cpu().numpy(), want)
     assert bad == 0, (bad, maxabs, ratio)
+
+
+@pytest.mark.parametrize("dist", [1, 2])
+def test_fixed_segments_overflow_falls_back_to_atomics(dist):
+    """A distant, narrow grid projects onto a handful of texels: their fixed segments (capacity =
+    the average over all texels) overflow by far, and the overflow is applied with atomics."""
+    w = small("cfg1_tiny", channels=16, roi_range=(38.0, 42.0, -1.0, 1.0, 0.5, 2.5), grid_size=(32, 32, 4),
+              depth_bins=64)
+    x = make_inputs(w, MODEL[dist], device="cuda", with_grad_out=True)
+    p = U.problem_for(x, w, dist, thr=0.0)
+    geo = c_oracle.geometry(x["projection_matrices"].cpu().numpy(), w.feat_hw, w.image_hw, list(w.roi_range),
+                            list(w.grid_size))
+    valid = geo["mask"].astype(bool)
+    texel = (geo["idx"][..., 2] * w.feat_hw[1] + geo["idx"][..., 0])[valid]          # (v0, u0) corner
+    per_texel = np.bincount(texel, minlength=w.feat_hw[0] * w.feat_hw[1])
+    seg_cap = capi.backward_max_pairs(p) // (w.feat_hw[0] * w.feat_hw[1] * 4)
+    assert seg_cap >= 16 and per_texel.max() > 8 * seg_cap, (seg_cap, per_texel.max())
+    check_all(w, x, dist, thr=0.0, modes=("gather", "gather_overwrite", "gather_counted"))
