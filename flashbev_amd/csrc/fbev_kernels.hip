@@ -1071,6 +1071,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
     for (int c0 = 0; c0 < k.C; c0 += span) {
         const int ch = c0 + lir * VEC;
         const bool on = worker_lane && ch < k.C;
+        const int ch_eff = on ? ch : 0, wslot_eff = min(wslot, wpw - 1);
         float acc[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
@@ -1083,11 +1084,12 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
             const int nb = min(kWave, wave_end - bstart);
             float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f);
             if (lane < nb) pr = *reinterpret_cast<const float4 *>(pairs + bstart + lane);
-            // a pair is written by the cell pass before this kernel starts; the range check
-            // only keeps a logic error from turning into a wild read
             const int word = __float_as_int(pr.x);
+            // a pair is written by the cell pass before this kernel starts; the range check only
+            // keeps a logic error from turning into a wild read (such a pair counts as cell 0
+            // with coefficient 0)
             const bool valid = (unsigned)(word >> bin_bits) < n_cells;
-            const int my_cell = valid ? (word >> bin_bits) : -1;
+            const int my_cell = valid ? (word >> bin_bits) : 0;
             const float my_coef = valid ? pr.y : 0.0f;
             if (c0 == 0 && valid) {
                 if (bin_sums) {
@@ -1099,31 +1101,35 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
                     sb += pr.w;
                 }
             }
+            // Full groups of UNR pairs per worker run without predicates (lanes that carry no
+            // channel gather channel 0 of some row and drop the result); the remainder goes one
+            // pair per worker.
             constexpr int UNR = 4;
-            for (int i = 0; i < nb; i += wpw * UNR) {
-                int cells[UNR];
+            const int group = wpw * UNR, full = nb - nb % group;
+            for (int i = 0; i < full; i += group) {
                 float coefs[UNR];
                 float g[UNR][VEC];
 #pragma unroll
                 for (int q = 0; q < UNR; ++q) {
-                    const int j = i + q * wpw + wslot;
-                    const int c = __shfl(my_cell, min(j, kWave - 1), kWave);
-                    coefs[q] = __shfl(my_coef, min(j, kWave - 1), kWave);
-                    cells[q] = (on && j < nb) ? c : -1;
+                    const int j = i + q * wpw + wslot_eff;
+                    const int c = __shfl(my_cell, j, kWave);
+                    coefs[q] = __shfl(my_coef, j, kWave);
+                    VecLoad<float, VEC>::ld(grad_out + (size_t)c * k.C + ch_eff, g[q]);
                 }
 #pragma unroll
-                for (int q = 0; q < UNR; ++q) {
-                    if (cells[q] >= 0) {
-                        const float *row = grad_out + (size_t)cells[q] * k.C + ch;
-                        VecLoad<float, VEC>::ld(row, g[q]);
-                    }
-                }
+                for (int q = 0; q < UNR; ++q)
 #pragma unroll
-                for (int q = 0; q < UNR; ++q) {
-                    if (cells[q] >= 0) {
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coefs[q], g[q][v], acc[v]);
+            }
+            for (int i = full; i < nb; i += wpw) {
+                const int j = i + wslot_eff;
+                const int c = __shfl(my_cell, min(j, kWave - 1), kWave);
+                const float coef = __shfl(my_coef, min(j, kWave - 1), kWave);
+                if (j < nb) {
+                    float g[VEC];
+                    VecLoad<float, VEC>::ld(grad_out + (size_t)c * k.C + ch_eff, g);
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coefs[q], g[q][v], acc[v]);
-                    }
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coef, g[v], acc[v]);
                 }
             }
         }
