@@ -21,7 +21,7 @@ parameters, tools/config/config.yaml:29).  The single JSON line printed on stdou
                         (oracle/dense_torch.py), forward+backward via autograd on the host
                         cores, same workload -- a reported baseline, not a target.
 ``--table`` additionally measures every configuration and depth model, forward and
-forward+backward, and writes the table to gpurun_out/bench_table.{json,md}.
+forward+backward, and writes the table to <--table-dir>/bench_table.{json,md}.
 """
 from __future__ import annotations
 
@@ -206,7 +206,7 @@ def stats(v):
             "p99": q(0.99)}
 
 
-def run_table(steps: int, warmup: int):
+def run_table(steps: int, warmup: int, out_dir: str):
     rows = []
     jobs = [("cfg1_tiny", None), ("cfg2_surround", None)]
     jobs += [("cfg3_zsweep", z) for z in (4, 8, 12, 16)]
@@ -231,10 +231,10 @@ def run_table(steps: int, warmup: int):
                   f"bwd {b_ms*1e3:9.1f} us ({rows[-1]['bwd_frac_hbm']*100:5.1f}% HBM)", file=sys.stderr, flush=True)
             del r
             torch.cuda.empty_cache()
-    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-    with open(os.path.join(ROOT, "gpurun_out", "bench_table.json"), "w") as fh:
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "bench_table.json"), "w") as fh:
         json.dump(rows, fh, indent=1)
-    with open(os.path.join(ROOT, "gpurun_out", "bench_table.md"), "w") as fh:
+    with open(os.path.join(out_dir, "bench_table.md"), "w") as fh:
         fh.write("| workload | depth model | dtype | fwd us | fwd GB/s | fwd % of 8 TB/s | bwd us | bwd GB/s | bwd % of 8 TB/s |\n")
         fh.write("|---|---|---|---|---|---|---|---|---|\n")
         for r_ in rows:
@@ -252,6 +252,7 @@ def main():
     ap.add_argument("--depth", default="laplace", choices=sorted(DIST_OF))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--table", action="store_true")
+    ap.add_argument("--table-dir", default="bench_out", help="directory (under the repository) for the --table files")
     ap.add_argument("--no-graph", action="store_true", help="time eagerly queued steps only")
     ap.add_argument("--backward-mode", type=int, default=0, choices=(0, 1, 2, 3),
                     help="0 auto (default), 1 atomic scatter, 2 inverse-map gather, 3 column owner")
@@ -328,7 +329,7 @@ def main():
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, args.depth)
     if args.table:
-        run_table(max(20, args.steps // 4), args.warmup)
+        run_table(max(20, args.steps // 4), args.warmup, os.path.join(ROOT, args.table_dir))
     print(json.dumps(line), flush=True)
 
 
