@@ -326,6 +326,19 @@ def main():
                      "forward": {"algorithmic_bytes": fb, "kernel_ms": fwd_k_ms,
                                  "frac": fb / fwd_k_ms / 1e6 / HBM_PEAK_GBS if fwd_k_ms else None}},
     }
+    # the same workload under the other depth models (the configuration text reads "D depth bins":
+    # that is the categorical model; the reference's own kernels only have the parametric ones)
+    others = {}
+    for name in sorted(DIST_OF):
+        if name == args.depth:
+            continue
+        r2 = Runner(w, name, backward_mode=args.backward_mode)
+        ms2, fwd2, bwd2 = time_steps(r2, args.steps, args.warmup, True)
+        others[name] = {"ms_per_step": ms2, "fwd_call_ms": statistics.mean(fwd2), "bwd_call_ms": statistics.mean(bwd2),
+                        "algorithmic_bytes_fwd_bwd": algorithmic_bytes(w, r2.model, False) + algorithmic_bytes(w, r2.model, True),
+                        "kept_samples": int(r2.counts.sum().item())}
+        del r2
+    line["other_depth_models"] = others
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, args.depth)
     if args.table:
