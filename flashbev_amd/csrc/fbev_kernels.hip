@@ -655,12 +655,29 @@ struct Pair {      // 16 bytes
 // Zero up to three regions of 32-bit words in one launch (segment counters and, when the
 // library is asked to, the two gradient buffers).  A kernel rather than hipMemsetAsync, so the
 // call can be captured in a HIP graph.
+// One thread clears one 16-byte unit of a region (its ragged head and tail word by word), so
+// the regions only have to be 4-byte aligned.
+__device__ __forceinline__ void zero_unit(int *p, long long n, long long unit) {
+    // units are counted from the first 16-byte boundary at or after p; unit 0 also takes the head
+    const long long head = (4 - (((uintptr_t)p >> 2) & 3)) & 3;      // words before the boundary
+    const long long first = unit * 4 + head;
+    if (unit == 0)
+        for (long long i = 0; i < head && i < n; ++i) p[i] = 0;
+    if (first + 4 <= n) {
+        *reinterpret_cast<int4 *>(p + first) = make_int4(0, 0, 0, 0);
+    } else {
+        for (long long i = first; i < n; ++i) p[i] = 0;
+    }
+}
+__host__ __device__ inline long long zero_units(long long n) { return n > 0 ? (n + 3) / 4 + 1 : 0; }
+
 __global__ __launch_bounds__(256) void fbev_fill_zero_kernel(int *a, long long na, int *b, long long nb, int *c,
                                                              long long nc) {
-    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < na) a[i] = 0;
-    else if (i < na + nb) b[i - na] = 0;
-    else if (i < na + nb + nc) c[i - na - nb] = 0;
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long ua = zero_units(na), ub = zero_units(nb), uc = zero_units(nc);
+    if (i < ua) zero_unit(a, na, i);
+    else if (i < ua + ub) zero_unit(b, nb, i - ua);
+    else if (i < ua + ub + uc) zero_unit(c, nc, i - ua - ub);
 }
 
 // Count, per (texel, replica), the sample corners that will contribute: phase A alone, with
@@ -1887,7 +1904,7 @@ int launch_zero(int *a, long long na, float *b, long long nb, float *c, long lon
     if (!a) na = 0;
     if (!b) nb = 0;
     if (!c) nc = 0;
-    const long long n = na + nb + nc;
+    const long long n = zero_units(na) + zero_units(nb) + zero_units(nc);
     if (n == 0) return FBEV_OK;
     prof::Scope timer(prof::kZero, st);
     hipLaunchKernelGGL(fbev_fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a, na,
