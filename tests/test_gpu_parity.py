@@ -135,3 +135,24 @@ def test_autograd_operator_matches_capi():
     want_dd, want_df = U.oracle_backward(x, w, 1)
     assert U.violations(f.grad.cpu().numpy(), want_df)[0] == 0
     assert U.violations(d.grad.cpu().numpy(), want_dd)[0] == 0
+
+
+@pytest.mark.parametrize("name,dist", [("gaussian", 0), ("laplace", 1), ("categorical", 2)])
+def test_kernels_against_the_committed_vectors(name, dist):
+    """The tiny configuration against tests/golden/ (the oracle's outputs, committed): masks,
+    indices, fractions and counts bit for bit, values within the fp32 tolerance."""
+    import os
+
+    want = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", f"cfg1_tiny_{name}.npz"))
+    w, x = _inputs("cfg1_tiny", dist)
+    mask, idx, frac = U.capi_geometry(x["projection_matrices"], w)
+    assert np.array_equal(mask.cpu().numpy(), want["mask"])
+    assert np.array_equal(idx.cpu().numpy().astype(np.int16), want["idx"])
+    assert np.array_equal(frac.cpu().numpy().view(np.uint32), want["frac"].view(np.uint32))
+    out, cnt = U.capi_forward(x, w, dist, with_count=True)
+    assert np.array_equal(cnt.cpu().numpy(), want["count"])
+    assert U.violations(out.cpu().numpy(), want["out"])[0] == 0
+    for mode in ("gather", "gather_counted", "scatter", "columns"):
+        dd, df = U.capi_backward(x, w, dist, mode=mode)
+        assert U.violations(df.cpu().numpy(), want["d_feats"])[0] == 0, mode
+        assert U.violations(dd.cpu().numpy(), want["d_depth"])[0] == 0, mode

@@ -308,3 +308,27 @@ def test_c_backward_vs_dense_autograd_on_surround_rig():
     dd_c, df_c = U.oracle_backward(x, w, 1)
     assert U.violations(df_c, df.numpy(), rtol=1e-3, atol=1e-5)[0] == 0
     assert U.violations(dd_c, dd.numpy(), rtol=2e-3, atol=2e-4)[0] == 0
+
+
+@pytest.mark.parametrize("name", ["gaussian", "laplace", "categorical"])
+def test_oracle_reproduces_the_committed_vectors(name):
+    """tests/golden/ holds the oracle's outputs for the tiny configuration (written by
+    tests/golden/make_fixtures.py): the seeded inputs still hash to what they were, and the
+    oracle still answers bit for bit the same."""
+    import importlib.util
+    import os
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(here, "make_fixtures.py"))
+    mf = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mf)
+    dist, model = mf.MODELS[name]
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, model, device="cpu", with_grad_out=True)
+    want = np.load(os.path.join(here, f"cfg1_tiny_{name}.npz"))
+    assert mf.input_digest(x) == str(want["digest"]), "the seeded inputs changed: regenerate the fixtures knowingly"
+    got = mf.oracle_outputs(w, x, dist)
+    for key in ("mask", "idx", "count"):
+        assert np.array_equal(got[key], want[key]), key
+    for key in ("frac", "out", "d_depth", "d_feats"):
+        assert np.array_equal(got[key].view(np.uint32), want[key].view(np.uint32)), key
