@@ -145,6 +145,8 @@ def test_kernels_against_the_committed_vectors(name, dist):
 
     want = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", f"cfg1_tiny_{name}.npz"))
     w, x = _inputs("cfg1_tiny", dist)
+    for key in ("image_feats", "depth_params", "projection_matrices", "grad_out"):      # the stored inputs
+        x[key] = torch.from_numpy(want[key]).cuda()
     mask, idx, frac = U.capi_geometry(x["projection_matrices"], w)
     assert np.array_equal(mask.cpu().numpy(), want["mask"])
     assert np.array_equal(idx.cpu().numpy().astype(np.int16), want["idx"])
