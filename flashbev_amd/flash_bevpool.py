@@ -44,6 +44,20 @@ def _backward_mode() -> int:
     if name not in _BACKWARD_MODES:
         raise ValueError(f"FLASHBEV_BACKWARD must be one of {sorted(_BACKWARD_MODES)}, got {name!r}")
     return _BACKWARD_MODES[name]
+
+
+def _pair_capacity(batch: int, cams: int, grid) -> int:
+    """Pair slots of the inverse-map workspace.  Room for every sample corner (16 bytes each)
+    lets the library skip its counting passes; FLASHBEV_WORKSPACE_MB (default 16384) bounds the
+    allocation, and a smaller workspace is packed exactly instead (-1 = the extension's default,
+    room for everything)."""
+    limit_mb = float(os.environ.get("FLASHBEV_WORKSPACE_MB", "16384"))
+    max_pairs = 4 * batch * cams * grid[0] * grid[1] * grid[2]
+    if max_pairs * 16 <= limit_mb * 2 ** 20:
+        return -1
+    return max(0, int(limit_mb * 2 ** 20) // 16)
+
+
 _host_cache: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()
 
 
@@ -140,6 +154,7 @@ class FlashBEVPool(torch.autograd.Function):
 
         ctx.save_for_backward(depth_params, image_feats, projection_matrices)
         ctx.counts = counts
+        ctx.pair_capacity = _pair_capacity(B, N, grid)
         ctx.host = (fs_host, image_t, roi_t, grid_t)
         ctx.total_threads = out.numel()
         ctx.depth_distribution = depth_distribution
@@ -168,7 +183,7 @@ class FlashBEVPool(torch.autograd.Function):
                 out_grad.contiguous().float(), depth_params, image_feats, projection_matrices,
                 fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
                 ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
-                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, -1, ctx.counts, False)
+                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, ctx.pair_capacity, ctx.counts, False)
         return (depth_params_grad, image_feats_grad) + (None,) * 14
 
 

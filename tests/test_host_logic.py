@@ -261,3 +261,11 @@ def test_latency_sweep_harness_selects_experiments_and_keeps_the_reference_schem
     assert set(stats) == {"latency_mean_ms", "latency_std_ms", "latency_min_ms", "latency_max_ms", "latency_p50_ms",
                           "latency_p95_ms", "latency_p99_ms"}
     assert stats["latency_mean_ms"] == 2.5 and stats["latency_p50_ms"] == 2.5
+
+
+def test_workspace_limit_selects_the_packed_layout(monkeypatch):
+    """Room for every sample corner by default; a bound in MB turns into a pair capacity."""
+    assert op_module._pair_capacity(1, 6, [128, 128, 8]) == -1
+    monkeypatch.setenv("FLASHBEV_WORKSPACE_MB", "16")
+    assert op_module._pair_capacity(1, 6, [128, 128, 8]) == 16 * 2 ** 20 // 16       # 50 MB would be needed
+    assert op_module._pair_capacity(1, 1, [32, 32, 4]) == -1
