@@ -8,6 +8,8 @@ Drop-in for the operator layer of yokosyun/FlashBEV's ``flashbevpool`` package
 from .flash_bevpool import FlashBEVPool, flash_bevpool, voxel_geometry
 from .rig import create_projection_matrix
 from .sampling_vt import SamplingVT
+from .sampling_vt_ops import sampling_vt_pillarpool_fused
 
-__all__ = ["FlashBEVPool", "flash_bevpool", "SamplingVT", "create_projection_matrix", "voxel_geometry"]
+__all__ = ["FlashBEVPool", "flash_bevpool", "SamplingVT", "sampling_vt_pillarpool_fused", "create_projection_matrix",
+           "voxel_geometry"]
 __version__ = "0.1.0"

@@ -33,6 +33,8 @@ def load_ext():
     spec.loader.exec_module(mod)
     # same module name as the reference's extension, so `import flashbevpool_ext` keeps working
     sys.modules.setdefault("flashbevpool_ext", mod)
+    # the reference keeps its PillarPool baseline in a second extension module; here one module serves both
+    sys.modules.setdefault("sampling_vt_ext", mod)
     _ext = mod
     return mod
 

@@ -17,7 +17,7 @@ FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
 EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_columns",
            "fbev_backward_columns_workspace_bytes", "fbev_backward_max_pairs",
-           "fbev_backward_workspace_bytes", "fbev_sample_geometry", "fbev_algorithmic_bytes",
+           "fbev_backward_workspace_bytes", "fbev_pillarpool_forward", "fbev_sample_geometry", "fbev_algorithmic_bytes",
            "fbev_profile_enable", "fbev_profile_kernel_count", "fbev_profile_kernel_name",
            "fbev_profile_collect", "fbev_status_string", "fbev_abi_version", "fbev_problem_size")
 
@@ -33,6 +33,14 @@ class FbevProblem(ctypes.Structure):
         ("depth_distribution", ctypes.c_int32), ("depth_bins", ctypes.c_int32),
         ("depth_min", ctypes.c_float), ("depth_step", ctypes.c_float),
         ("in_dtype", ctypes.c_int32), ("reduction", ctypes.c_int32), ("proj_stride", ctypes.c_int32),
+    ]
+
+
+class FbevPillarProblem(ctypes.Structure):
+    _fields_ = [
+        ("channels", ctypes.c_int32), ("n_intervals", ctypes.c_int32), ("batch", ctypes.c_int32),
+        ("num_cams", ctypes.c_int32), ("feat_h", ctypes.c_int32), ("feat_w", ctypes.c_int32),
+        ("epsilon", ctypes.c_float), ("depth_distribution", ctypes.c_int32),
     ]
 
 
@@ -58,6 +66,8 @@ def load() -> ctypes.CDLL:
         lib.fbev_backward_max_pairs.restype = ctypes.c_uint64
         lib.fbev_backward_workspace_bytes.argtypes = [pp, ctypes.c_uint64]
         lib.fbev_backward_workspace_bytes.restype = ctypes.c_size_t
+        lib.fbev_pillarpool_forward.argtypes = [ctypes.POINTER(FbevPillarProblem)] + [vp] * 11
+        lib.fbev_pillarpool_forward.restype = ctypes.c_int
         lib.fbev_sample_geometry.argtypes = [pp, vp, vp, vp, vp, vp]
         lib.fbev_sample_geometry.restype = ctypes.c_int
         lib.fbev_algorithmic_bytes.argtypes = [pp, ctypes.c_int]
@@ -156,6 +166,13 @@ def backward_max_pairs(p: FbevProblem) -> int:
 
 def backward_workspace_bytes(p: FbevProblem, pair_capacity: int) -> int:
     return int(load().fbev_backward_workspace_bytes(ctypes.byref(p), ctypes.c_uint64(int(pair_capacity))))
+
+
+def pillarpool_forward(p: FbevPillarProblem, depth_ptr, feats_ptr, u_ptr, v_ptr, z_ptr, batch_camera_ptr, ranks_ptr,
+                       starts_ptr, lengths_ptr, out_ptr, stream: int = 0) -> int:
+    return load().fbev_pillarpool_forward(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(u_ptr), _p(v_ptr),
+                                          _p(z_ptr), _p(batch_camera_ptr), _p(ranks_ptr), _p(starts_ptr),
+                                          _p(lengths_ptr), _p(out_ptr), _p(stream))
 
 
 def sample_geometry(p: FbevProblem, proj_ptr: int, mask_ptr: Optional[int], idx_ptr: Optional[int],

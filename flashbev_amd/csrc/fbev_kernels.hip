@@ -39,12 +39,13 @@ namespace {
 // call count per kernel.  Disabled (the default) it costs one relaxed atomic load per launch.
 namespace prof {
 enum Kid { kForward, kBackwardScatter, kZero, kCount, kScanChunks, kScanSums, kBackwardCells, kBackwardTexel,
-           kGeometry, kBackwardColumn, kCellCount, kNum };
+           kGeometry, kBackwardColumn, kCellCount, kPillar, kNum };
 const char *const kNames[kNum] = {"fbev_forward_kernel", "fbev_backward_cells_kernel<scatter>",
                                   "fbev_fill_zero_kernel", "fbev_count_kernel", "fbev_scan_chunks_kernel",
                                   "fbev_scan_sums_kernel", "fbev_backward_cells_kernel<fill>",
                                   "fbev_backward_texel_kernel", "fbev_geometry_kernel",
-                                  "fbev_backward_column_kernel", "fbev_forward_kernel<count only>"};
+                                  "fbev_backward_column_kernel", "fbev_forward_kernel<count only>",
+                                  "fbev_pillar_kernel"};
 struct Rec { hipEvent_t a, b; int kid; };
 std::atomic<bool> enabled{false};
 std::mutex mu;
@@ -1654,6 +1655,81 @@ __global__ __launch_bounds__(kColThreads) void fbev_backward_column_kernel(
         column_consume<T, VEC>(k, cp, L, n_ent, u, rowbase, first_flush, grad_out, feats, d_depth, d_feats);
 }
 
+// ---------------------------------------------------------------- interval pooling (baseline)
+// The reference's second method ("Sampling-VT + PillarPool"): the host projects every sample,
+// keeps those in view, sorts them by BEV cell and hands over per-sample feature-map coordinates
+// plus one (start, length) interval per touched cell.  Lanes = (interval, channel vector): the
+// lanes of a slot walk their interval together; bilinear weights and the depth likelihood are
+// evaluated by every lane of the slot (cheap beside the four row gathers).  No weight threshold;
+// the mean runs over the samples that pass the kernel's own in-view test.
+template <int VEC>
+__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_pillar_kernel(
+    int C, int n_intervals, int H, int W, int lanes_per_slot, float eps, int laplace,
+    const float *__restrict__ depth, const float *__restrict__ feats, const float *__restrict__ u_coords,
+    const float *__restrict__ v_coords, const float *__restrict__ z_coords, const int *__restrict__ batch_camera,
+    const int *__restrict__ ranks_bev, const int *__restrict__ interval_starts,
+    const int *__restrict__ interval_lengths, float *__restrict__ out) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+    const int slots = kWave / lanes_per_slot;
+    const int slot = lane / lanes_per_slot, lis = lane - slot * lanes_per_slot;
+    const long long interval = ((long long)blockIdx.x * kWavesPerBlock + wave) * slots + slot;
+    if (slot >= slots || interval >= n_intervals) return;
+    const int start = interval_starts[interval], len = interval_lengths[interval];
+    const float Wf = (float)W, Hf = (float)H;
+    const int span = lanes_per_slot * VEC;
+    float *o = out + (size_t)ranks_bev[start] * C;
+    for (int c0 = 0; c0 < C; c0 += span) {
+        const int ch = c0 + lis * VEC;
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+        int count = 0;
+        for (int i = 0; i < len; ++i) {
+            const float fu = u_coords[start + i], fv = v_coords[start + i], d = z_coords[start + i];
+            if (!(fu >= 0.0f && fu < Wf && fv >= 0.0f && fv < Hf && d > 0.0f)) continue;
+            const float u0f = floorf(fu), v0f = floorf(fv);
+            const int u0 = (int)u0f, v0 = (int)v0f;
+            const int u1 = min(u0 + 1, W - 1), v1 = min(v0 + 1, H - 1);
+            const float du = fu - u0f, dv = fv - v0f;
+            const float w00 = (1.0f - du) * (1.0f - dv), w01 = (1.0f - du) * dv, w10 = du * (1.0f - dv), w11 = du * dv;
+            const size_t base = (size_t)batch_camera[start + i] * H * W;
+            const size_t t00 = base + (size_t)v0 * W + u0, t01 = base + (size_t)v1 * W + u0;
+            const size_t t10 = base + (size_t)v0 * W + u1, t11 = base + (size_t)v1 * W + u1;
+            const float2 p00 = *reinterpret_cast<const float2 *>(depth + t00 * 2);
+            const float2 p01 = *reinterpret_cast<const float2 *>(depth + t01 * 2);
+            const float2 p10 = *reinterpret_cast<const float2 *>(depth + t10 * 2);
+            const float2 p11 = *reinterpret_cast<const float2 *>(depth + t11 * 2);
+            const float mu = bilerp(w00, w01, w10, w11, p00.x, p01.x, p10.x, p11.x);
+            const float s = bilerp(w00, w01, w10, w11, p00.y, p01.y, p10.y, p11.y) + eps;
+            const float zs = (d - mu) / s;
+            const float wgt = laplace ? (0.5f * expf(-fabsf(zs))) / s : expf((-0.5f * zs) * zs) / s;
+            ++count;
+            if (ch < C) {
+                float f00[VEC], f01[VEC], f10[VEC], f11[VEC];
+                VecLoad<float, VEC>::ld(feats + t00 * C + ch, f00);
+                VecLoad<float, VEC>::ld(feats + t01 * C + ch, f01);
+                VecLoad<float, VEC>::ld(feats + t10 * C + ch, f10);
+                VecLoad<float, VEC>::ld(feats + t11 * C + ch, f11);
+                const float a00 = w00 * wgt, a01 = w01 * wgt, a10 = w10 * wgt, a11 = w11 * wgt;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    float a = acc[v];
+                    a = __builtin_fmaf(a00, f00[v], a);
+                    a = __builtin_fmaf(a01, f01[v], a);
+                    a = __builtin_fmaf(a10, f10[v], a);
+                    a = __builtin_fmaf(a11, f11[v], a);
+                    acc[v] = a;
+                }
+            }
+        }
+        if (ch < C) {
+            const float nf = (float)count;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) o[ch + v] = count > 0 ? acc[v] / nf : 0.0f;
+        }
+    }
+}
+
 // ---------------------------------------------------------------- geometry inspection
 __global__ __launch_bounds__(256) void fbev_geometry_kernel(KParams k, const float *__restrict__ proj,
                                                             uint8_t *mask, int32_t *idx, float *frac,
@@ -2106,6 +2182,45 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     else
         hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels, n_split), dim3(kWave * kWavesPerBlock), lds,
                            st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+int fbev_pillarpool_forward(const fbev_pillar_problem *p, const float *depth, const float *feats,
+                            const float *u_coords, const float *v_coords, const float *z_coords,
+                            const int32_t *batch_camera, const int32_t *ranks_bev, const int32_t *interval_starts,
+                            const int32_t *interval_lengths, float *out, void *stream) {
+    if (!p) return FBEV_ERR_NULL;
+    if (p->channels <= 0 || p->n_intervals < 0 || p->batch <= 0 || p->num_cams <= 0 || p->feat_h <= 0 || p->feat_w <= 0)
+        return FBEV_ERR_SHAPE;
+    if (p->depth_distribution != FBEV_GAUSSIAN && p->depth_distribution != FBEV_LAPLACE) return FBEV_ERR_UNSUPPORTED;
+    if (p->n_intervals == 0) return FBEV_OK;
+    if (!depth || !feats || !u_coords || !v_coords || !z_coords || !batch_camera || !ranks_bev || !interval_starts ||
+        !interval_lengths || !out)
+        return FBEV_ERR_NULL;
+    if ((uintptr_t)depth % 8 || (uintptr_t)feats % 4 || (uintptr_t)u_coords % 4 || (uintptr_t)v_coords % 4 ||
+        (uintptr_t)z_coords % 4 || (uintptr_t)batch_camera % 4 || (uintptr_t)ranks_bev % 4 ||
+        (uintptr_t)interval_starts % 4 || (uintptr_t)interval_lengths % 4 || (uintptr_t)out % 4)
+        return FBEV_ERR_ALIGNMENT;
+    if ((long long)p->batch * p->num_cams * p->feat_h * p->feat_w >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    const bool vec4 = p->channels % 4 == 0 && (uintptr_t)feats % 16 == 0;
+    const int vec = vec4 ? 4 : 1;
+    const int cq = (p->channels + vec - 1) / vec;
+    const int lps = cq < kWave ? cq : kWave;
+    const int per_block = (kWave / lps) * kWavesPerBlock;
+    const long long blocks = ((long long)p->n_intervals + per_block - 1) / per_block;
+    if (blocks >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    prof::Scope timer(prof::kPillar, st);
+    if (vec4)
+        hipLaunchKernelGGL((fbev_pillar_kernel<4>), dim3((unsigned)blocks), dim3(kWave * kWavesPerBlock), 0, st,
+                           p->channels, p->n_intervals, p->feat_h, p->feat_w, lps, p->epsilon,
+                           p->depth_distribution == FBEV_LAPLACE ? 1 : 0, depth, feats, u_coords, v_coords, z_coords,
+                           batch_camera, ranks_bev, interval_starts, interval_lengths, out);
+    else
+        hipLaunchKernelGGL((fbev_pillar_kernel<1>), dim3((unsigned)blocks), dim3(kWave * kWavesPerBlock), 0, st,
+                           p->channels, p->n_intervals, p->feat_h, p->feat_w, lps, p->epsilon,
+                           p->depth_distribution == FBEV_LAPLACE ? 1 : 0, depth, feats, u_coords, v_coords, z_coords,
+                           batch_camera, ranks_bev, interval_starts, interval_lengths, out);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 

@@ -300,6 +300,52 @@ std::vector<at::Tensor> sample_geometry(const at::Tensor &projection_matrices, i
     return {mask, idx, frac};
 }
 
+// Same positional order as the reference's sampling_vt_pillarpool_fused_forward
+// (flashbev/flashbevpool/src/sampling_vt.cpp:13-52): note interval_lengths before
+// interval_starts.  All tensors on one device, contiguous; float32 / int32 as in the reference.
+void sampling_vt_pillarpool_fused_forward(const at::Tensor &depth, const at::Tensor &feat, const at::Tensor &u_coords,
+                                          const at::Tensor &v_coords, const at::Tensor &z_coords,
+                                          const at::Tensor &batch_camera_indices, const at::Tensor &ranks_bev,
+                                          const at::Tensor &interval_lengths, const at::Tensor &interval_starts,
+                                          at::Tensor out, int batch_size, int num_cameras, int feat_h, int feat_w,
+                                          float epsilon, int depth_distribution) {
+    TORCH_CHECK(feat.is_cuda(), "sampling_vt_pillarpool_fused_forward: feat must be on a ROCm GPU");
+    const at::Tensor *all[] = {&depth, &u_coords, &v_coords, &z_coords, &batch_camera_indices, &ranks_bev,
+                               &interval_lengths, &interval_starts, &out};
+    for (const at::Tensor *t : all) check_dev(*t, feat, "an argument");
+    for (const at::Tensor *t : {&depth, &feat, &u_coords, &v_coords, &z_coords, (const at::Tensor *)&out})
+        TORCH_CHECK(t->scalar_type() == at::kFloat && t->is_contiguous(),
+                    "sampling_vt_pillarpool_fused_forward: float tensors must be contiguous float32");
+    for (const at::Tensor *t : {&batch_camera_indices, &ranks_bev, &interval_lengths, &interval_starts})
+        TORCH_CHECK(t->scalar_type() == at::kInt && t->is_contiguous(),
+                    "sampling_vt_pillarpool_fused_forward: index tensors must be contiguous int32");
+    TORCH_CHECK(feat.dim() == 5 && feat.size(0) == batch_size && feat.size(1) == num_cameras && feat.size(2) == feat_h &&
+                    feat.size(3) == feat_w,
+                "sampling_vt_pillarpool_fused_forward: feat must be [B,N,H,W,C], got ", feat.sizes());
+    TORCH_CHECK(depth.numel() == (int64_t)batch_size * num_cameras * feat_h * feat_w * 2,
+                "sampling_vt_pillarpool_fused_forward: depth must be [B,N,H,W,2], got ", depth.sizes());
+    const int64_t n = u_coords.numel();
+    TORCH_CHECK(v_coords.numel() == n && z_coords.numel() == n && batch_camera_indices.numel() == n &&
+                    ranks_bev.numel() == n,
+                "sampling_vt_pillarpool_fused_forward: per-sample tensors must have the same length");
+    TORCH_CHECK(interval_starts.numel() == interval_lengths.numel(),
+                "sampling_vt_pillarpool_fused_forward: interval_starts and interval_lengths differ in length");
+    TORCH_CHECK(out.size(-1) == feat.size(4), "sampling_vt_pillarpool_fused_forward: out's last dimension must be C");
+    fbev_pillar_problem p = {};
+    p.channels = (int32_t)feat.size(4);
+    p.n_intervals = (int32_t)interval_lengths.numel();
+    p.batch = batch_size; p.num_cams = num_cameras; p.feat_h = feat_h; p.feat_w = feat_w;
+    p.epsilon = epsilon; p.depth_distribution = depth_distribution;
+    DeviceScope scope(feat.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(feat.get_device()).stream();
+    raise_on(fbev_pillarpool_forward(&p, depth.data_ptr<float>(), feat.data_ptr<float>(), u_coords.data_ptr<float>(),
+                                     v_coords.data_ptr<float>(), z_coords.data_ptr<float>(),
+                                     batch_camera_indices.data_ptr<int>(), ranks_bev.data_ptr<int>(),
+                                     interval_starts.data_ptr<int>(), interval_lengths.data_ptr<int>(),
+                                     out.data_ptr<float>(), st),
+             "fbev_pillarpool_forward");
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     namespace py = pybind11;
     m.def("flash_bevpool_forward", &flash_bevpool_forward, "fused camera->BEV pooling, forward",
@@ -321,5 +367,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("sample_geometry", &sample_geometry, "per-sample validity mask and corner indices (parity hook)",
           py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
           py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);
+    m.def("sampling_vt_pillarpool_fused_forward", &sampling_vt_pillarpool_fused_forward,
+          "interval pooling over precomputed sample lists (the reference's PillarPool baseline)");
     m.def("abi_version", []() { return fbev_abi_version(); });
 }

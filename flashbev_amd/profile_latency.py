@@ -16,8 +16,9 @@ operator on generated tensors like ``benchmark_flashbevpool_kernel``
 with the host clock, allocation of the output included, as the reference does.  ``--backward``
 adds a forward+backward record per point (the reference never times its backward).
 
-Only this package's method exists here; the reference's dense PyTorch and PillarPool rows have
-no counterpart.
+``--module --with-baseline`` adds the reference's "Sampling-VT+PillarPool" method (projection
+and sorting in PyTorch, interval pooling kernel); its dense PyTorch method has no counterpart
+here.
 """
 from __future__ import annotations
 
@@ -35,6 +36,7 @@ from .sampling_vt import SamplingVT
 from .workloads import SURROUND_YAWS
 
 METHOD = "FlashBEV(ours)"
+BASELINE_METHOD = "Sampling-VT+PillarPool"
 
 
 def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
@@ -65,6 +67,8 @@ def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
     mode.add_argument("--kernel-only", dest="kernel_only", action="store_true", default=True)
     mode.add_argument("--module", dest="kernel_only", action="store_false")
     ap.add_argument("--backward", action="store_true")
+    ap.add_argument("--with-baseline", action="store_true",
+                    help="module mode: also time the Sampling-VT+PillarPool method (forward only)")
     ap.add_argument("--device", default="cuda")
     ap.add_argument("--output-json", default=None)
     return ap.parse_args(argv)
@@ -172,6 +176,19 @@ def run_point(args: argparse.Namespace, num_bins: int, num_cams: int, threshold:
                 return vt(inp)
 
         records.append({**base, "pass": "forward", **time_calls(forward, args.num_warmup, args.num_iterations)})
+        if args.with_baseline:
+            other = SamplingVT(grid, (args.input_h, args.input_w), downsample=args.downsample,
+                               in_channels=args.in_channels, out_channels=args.out_channels, fuse_projection=False,
+                               use_bev_pool=True, depth_distribution=args.depth_distribution).to(dev).eval()
+            other.load_state_dict(vt.state_dict(), strict=False)
+
+            def forward_baseline():
+                with torch.no_grad():
+                    return other(inp)
+
+            records.append({**base, "method": BASELINE_METHOD, "fuse_projection": False, "use_bev_pool": True,
+                            "pass": "forward", **time_calls(forward_baseline, args.num_warmup, args.num_iterations)})
+            del other
         if args.backward:
             vt.train()
 

@@ -13,8 +13,11 @@ every call (sampling_vt.py:252-253, flash_bevpool.py:47-48) does not exist here,
 memory format of the incoming feature map; the ``[B, C, Y, X]`` result is a view of the
 operator's ``[B, Y, X, C]`` output (channels-last memory format), not a copy.
 
-Only the fused path exists here: ``fuse_projection=False`` (the reference's dense PyTorch and
-PillarPool branches, sampling_vt.py:269-292) raises.  Grid sizes are rounded, not truncated
+Besides the fused path there is the reference's baseline method
+(``fuse_projection=False, use_bev_pool=True``, sampling_vt.py:269-281,296-447): every sample is
+projected with PyTorch operations, masked, sorted by BEV cell, and pooled by
+``sampling_vt_pillarpool_fused``.  The dense PyTorch branch
+(``fuse_projection=False, use_bev_pool=False``, sampling_vt.py:282-292) raises.  Grid sizes are rounded, not truncated
 (the reference's float-to-int32 truncation at sampling_vt.py:189-193 can lose a cell when
 (hi - lo) / step lands just below an integer).
 """
@@ -26,6 +29,7 @@ import torch.nn.functional as F
 
 from .flash_bevpool import flash_bevpool
 from .rig import create_projection_matrix
+from .sampling_vt_ops import sampling_vt_pillarpool_fused
 
 
 class SamplingVT(nn.Module):
@@ -34,10 +38,10 @@ class SamplingVT(nn.Module):
                  depth_distribution="laplace", optimize_z_precompute=True, use_warp_kernel=False,
                  use_vectorized_load=False, depth_weight_threshold=0.0):
         super().__init__()
-        if not fuse_projection:
+        if not fuse_projection and not use_bev_pool:
             raise NotImplementedError(
-                "SamplingVT: only the fused path (fuse_projection=True) is implemented; the dense "
-                "PyTorch and PillarPool branches of the reference are not part of this package")
+                "SamplingVT: the dense PyTorch branch of the reference (fuse_projection=False, "
+                "use_bev_pool=False) is not part of this package")
         self.depth_distribution = depth_distribution.lower()
         if self.depth_distribution not in ("laplace", "gaussian"):
             raise ValueError(f"depth_distribution must be 'laplace' or 'gaussian', got '{depth_distribution}'")
@@ -65,6 +69,10 @@ class SamplingVT(nn.Module):
         # host copies: the operator then never reads sizes back from the device
         self._roi_host = [float(v) for a in axes for v in a[:2]]
         self._grid_host = sizes
+        if not fuse_projection:
+            # voxel centres [X, Y, Z, 3] of the baseline method (sampling_vt.py:364-378)
+            centres = [torch.linspace(a[0], a[1], n + 1)[:-1] + (a[1] - a[0]) / n / 2.0 for a, n in zip(axes, sizes)]
+            self.register_buffer("coords_3d", torch.stack(torch.meshgrid(*centres, indexing="ij"), dim=-1))
 
     @staticmethod
     def _pointwise(conv, x):
@@ -89,12 +97,45 @@ class SamplingVT(nn.Module):
         x = x.reshape(B * N, C, H, W)
         features_last = self._pointwise(self.context_network, x)     # [B*N, H, W, C_out]
         depths_last = self._depth_last(x)                            # [B*N, H, W, 2]
-        bev = self._pool(input, features_last, depths_last)
+        pool = self._pool if self.fuse_projection else self._pool_sorted_lists
+        bev = pool(input, features_last, depths_last)
         return bev, depths_last.movedim(-1, 1)
 
     def sampling_vt(self, input, features_pv, depths):
         """Reference entry point with channels-first maps ``[B*N, C, H, W]`` / ``[B*N, 2, H, W]``."""
-        return self._pool(input, features_pv.movedim(-3, -1), depths.movedim(-3, -1))
+        pool = self._pool if self.fuse_projection else self._pool_sorted_lists
+        return pool(input, features_pv.movedim(-3, -1), depths.movedim(-3, -1))
+
+    def _pool_sorted_lists(self, input, features_last, depths_last):
+        """The baseline method: project all voxel centres, keep the samples in view, sort them by
+        BEV cell and pool the lists (sampling_vt.py:269-281, 296-447)."""
+        B, N = input[3].shape[:2]
+        P = create_projection_matrix(*input[1:7])                              # [B, N, 3, 4]
+        H, W = features_last.shape[1:3]
+        X, Y, Z = self._grid_host
+        xyz1 = torch.cat([self.coords_3d, torch.ones_like(self.coords_3d[..., :1])], dim=-1)   # [X, Y, Z, 4]
+        uvd = torch.einsum("bnij,xyzj->bnxyzi", P, xyz1)                      # homogeneous image coordinates
+        d = uvd[..., 2]
+        eps = 1e-6
+        dc = torch.where(d >= 0, d.clamp(min=eps), d.clamp(max=-eps))         # sampling_vt.py:449-466
+        fu = uvd[..., 0] / dc / self.image_size[1] * W
+        fv = uvd[..., 1] / dc / self.image_size[0] * H
+        in_view = (fu >= 0) & (fu < W) & (fv >= 0) & (fv < H) & (d > 0)        # [B, N, X, Y, Z]
+        cell = torch.arange(B * X * Y, device=d.device).view(B, 1, X, Y, 1).expand(B, N, X, Y, Z)[in_view]
+        camera = torch.arange(B * N, device=d.device).view(B, N, 1, 1, 1).expand(B, N, X, Y, Z)[in_view]
+        cell, order = torch.sort(cell)
+        first = torch.ones_like(cell, dtype=torch.bool)
+        first[1:] = cell[1:] != cell[:-1]
+        starts = torch.nonzero(first).flatten()
+        lengths = torch.diff(starts, append=starts.new_tensor([cell.numel()]))
+        bev = sampling_vt_pillarpool_fused(
+            depth=depths_last.unflatten(0, (B, N)), feat=features_last.unflatten(0, (B, N)),
+            u_coords=fu[in_view][order], v_coords=fv[in_view][order], z_coords=d[in_view][order],
+            batch_camera_indices=camera[order], ranks_bev=cell,
+            bev_feat_shape=(B, X, Y, 1, features_last.shape[-1]), interval_starts=starts, interval_lengths=lengths,
+            batch_size=B, num_cameras=N, feat_h=H, feat_w=W, epsilon=1e-6,
+            depth_distribution=1 if self.depth_distribution == "laplace" else 0)      # [B, C, X, Y, 1]
+        return bev.squeeze(-1).movedim(-1, -2)                                        # [B, C, Y, X]
 
     def _pool(self, input, features_last, depths_last):
         B, N = input[3].shape[:2]

@@ -150,6 +150,36 @@ uint64_t fbev_backward_max_pairs(const fbev_problem *p);
 size_t fbev_backward_workspace_bytes(const fbev_problem *p, uint64_t pair_capacity);
 
 /*
+ * The reference's baseline method "Sampling-VT + PillarPool": pooling over precomputed,
+ * cell-sorted sample lists.  The caller has projected every (cell, camera, height) sample,
+ * kept those in view and sorted them by BEV cell; sample s has feature-map coordinates
+ * (u_coords[s], v_coords[s]) in texels, depth z_coords[s] and camera
+ * batch_camera[s] = b * num_cams + n; interval i covers samples
+ * [interval_starts[i], interval_starts[i] + interval_lengths[i]) of one cell, whose output row
+ * is out[ranks_bev[interval_starts[i]] * channels ...].  Each row receives the mean over its
+ * in-view samples of the bilinearly sampled features times the Gaussian / Laplace depth
+ * likelihood (no weight threshold); rows no interval names are left untouched (the caller
+ * zero-fills `out`).  fp32 only: depth [B,N,H,W,2], feats [B,N,H,W,C] channels-last.
+ * Replaces sampling_vt_pillarpool_fused(...)
+ * (flashbev/flashbevpool/src/sampling_vt_cuda.cu:131-148, kernel :24-129).
+ */
+typedef struct fbev_pillar_problem {
+    int32_t channels;    /* C */
+    int32_t n_intervals; /* touched cells */
+    int32_t batch;       /* B */
+    int32_t num_cams;    /* N */
+    int32_t feat_h;      /* H */
+    int32_t feat_w;      /* W */
+    float epsilon;       /* added to sigma */
+    int32_t depth_distribution; /* FBEV_GAUSSIAN / FBEV_LAPLACE */
+} fbev_pillar_problem;
+
+int fbev_pillarpool_forward(const fbev_pillar_problem *p, const float *depth, const float *feats,
+                            const float *u_coords, const float *v_coords, const float *z_coords,
+                            const int32_t *batch_camera, const int32_t *ranks_bev, const int32_t *interval_starts,
+                            const int32_t *interval_lengths, float *out, void *stream);
+
+/*
  * Inspection hook for parity tests: per (b, y, x, camera, height-bin) sample, in that
  * order, the projection validity and the bilinear corner indices the kernels use.
  *   mask  uint8  [B,gy,gx,N,gz]      1 = depth > 0 and inside the feature map

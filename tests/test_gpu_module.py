@@ -38,7 +38,9 @@ def test_module_state_dict_names_and_buffers():
     with pytest.raises(ValueError):
         SamplingVT(GRID, (256, 704), depth_distribution="uniform")
     with pytest.raises(NotImplementedError):
-        SamplingVT(GRID, (256, 704), fuse_projection=False)
+        SamplingVT(GRID, (256, 704), fuse_projection=False, use_bev_pool=False)
+    assert SamplingVT(GRID, (256, 704), in_channels=8, out_channels=4, fuse_projection=False).coords_3d.shape == \
+        (100, 100, 12, 3)
     # a step that divides the range only up to rounding still yields the intended count
     g2 = dict(GRID, z=[-5.0, 3.0, 8.0 / 12.0])
     assert SamplingVT(g2, (256, 704), in_channels=8, out_channels=4).sample_grid_size.tolist()[2] == 12
@@ -141,3 +143,66 @@ def test_forward_and_backward_replay_from_a_hip_graph():
         assert torch.allclose(feats.grad, want_f, rtol=1e-4, atol=1e-5), f"replay {i}: d_feats differs"
         assert torch.allclose(depth.grad, want_d, rtol=1e-4, atol=1e-5), f"replay {i}: d_depth differs"
         (feats.detach() * 2).sum().item()      # eager work and a host sync between replays
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dist,channels", [(0, 80), (1, 80), (1, 13)])
+def test_interval_pooling_baseline_matches_the_oracle(dist, channels):
+    """sampling_vt_pillarpool_fused on sample lists built from the oracle's own geometry equals
+    the oracle's forward without a weight threshold (the baseline has none)."""
+    import dataclasses
+
+    from flashbev_amd import sampling_vt_pillarpool_fused
+    from flashbev_amd.workloads import WORKLOADS, make_inputs
+    from oracle import c_oracle
+
+    w = dataclasses.replace(WORKLOADS["cfg2_surround"], channels=channels, grid_size=(40, 36, 5), batch=2)
+    x = make_inputs(w, "parametric", device="cpu")
+    B, N, (H, W), (gx, gy, gz) = w.batch, w.num_cams, w.feat_hw, w.grid_size
+    geo = c_oracle.geometry(x["projection_matrices"].numpy(), w.feat_hw, w.image_hw, list(w.roi_range), list(w.grid_size))
+    valid = geo["mask"].astype(bool)                                   # [B, gy, gx, N, gz]
+    fu = geo["idx"][..., 0].astype(np.float32) + geo["frac"][..., 0]
+    fv = geo["idx"][..., 2].astype(np.float32) + geo["frac"][..., 1]
+    b, iy, ix, n, _ = np.nonzero(valid)
+    rank = (b * gx + ix) * gy + iy                                     # output rows laid out [B, X, Y]
+    order = np.argsort(rank, kind="stable")
+    rank_s = rank[order]
+    first = np.ones(rank_s.size, dtype=bool)
+    first[1:] = rank_s[1:] != rank_s[:-1]
+    starts = np.nonzero(first)[0]
+    lengths = np.diff(np.append(starts, rank_s.size))
+    dev = "cuda"
+    t = lambda a, dt: torch.from_numpy(np.ascontiguousarray(a)).to(dev, dt)
+    out = sampling_vt_pillarpool_fused(
+        depth=x["depth_params"].to(dev), feat=x["image_feats"].to(dev),
+        u_coords=t(fu[valid][order], torch.float32), v_coords=t(fv[valid][order], torch.float32),
+        z_coords=t(geo["depth"][valid][order], torch.float32),
+        batch_camera_indices=t((b * N + n)[order], torch.int32), ranks_bev=t(rank_s, torch.int32),
+        bev_feat_shape=(B, gx, gy, 1, channels), interval_starts=t(starts, torch.int32),
+        interval_lengths=t(lengths, torch.int32), batch_size=B, num_cameras=N, feat_h=H, feat_w=W,
+        epsilon=1e-6, depth_distribution=dist)
+    assert out.shape == (B, channels, gx, gy, 1)
+    want = c_oracle.forward(x["depth_params"].numpy(), x["image_feats"].numpy(), x["projection_matrices"].numpy(),
+                            image_size=w.image_hw, roi_range=w.roi_range, grid_size=w.grid_size,
+                            depth_distribution=dist, depth_weight_threshold=0.0)              # [B, gy, gx, C]
+    got = out.squeeze(-1).permute(0, 3, 2, 1).cpu().numpy()                                   # [B, gy, gx, C]
+    bad, maxabs, ratio = U.violations(got, want)
+    assert bad == 0, (bad, maxabs, ratio)
+
+
+@pytest.mark.gpu
+def test_module_baseline_branch_agrees_with_the_fused_branch():
+    """fuse_projection=False, use_bev_pool=True (projection and sorting in PyTorch, then interval
+    pooling) against the fused operator with the same weights, by the reference's acceptance
+    statistics; the two differ only where a sample sits within rounding of the image border."""
+    vt, inp, _ = make_module_and_input("laplace", "cuda")
+    torch.manual_seed(42)
+    base = SamplingVT(GRID, (256, 704), downsample=16, in_channels=32, out_channels=24, fuse_projection=False,
+                      use_bev_pool=True, depth_distribution="laplace").to("cuda").eval()
+    base.load_state_dict(vt.state_dict(), strict=False)
+    with torch.no_grad():
+        a, _ = vt(inp)
+        b, _ = base(inp)
+    assert a.shape == b.shape == (1, 24, 100, 100)
+    m = U.reference_metrics(b.cpu().numpy(), a.cpu().numpy())
+    assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["mean_rel"] < 1e-3 and m["cosine"] > 0.9999, m
