@@ -206,3 +206,45 @@ def test_module_baseline_branch_agrees_with_the_fused_branch():
     assert a.shape == b.shape == (1, 24, 100, 100)
     m = U.reference_metrics(b.cpu().numpy(), a.cpu().numpy())
     assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["mean_rel"] < 1e-3 and m["cosine"] > 0.9999, m
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_half_precision_leaves_get_gradients_in_their_dtype(dtype):
+    """Half inputs go into the kernels as they are; the fp32 gradient buffers are cast to the
+    leaves' dtype by autograd and agree with the fp32 run to half precision."""
+    from flashbev_amd import flash_bevpool
+    from flashbev_amd.workloads import WORKLOADS, make_inputs
+
+    w = WORKLOADS["cfg2_surround"]
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    kw = dict(projection_matrices=x["projection_matrices"], feature_size=x["feature_size"],
+              image_size=list(w.image_hw), roi_range=list(w.roi_range), grid_size=list(w.grid_size),
+              depth_distribution=1)
+    grads = {}
+    for dt in (torch.float32, dtype):
+        # the same (half-representable) values in both runs
+        f = x["image_feats"].to(dtype).to(dt).requires_grad_(True)
+        d = x["depth_params"].to(dtype).to(dt).requires_grad_(True)
+        out = flash_bevpool(image_feats=f, depth_params=d, **kw)
+        assert out.dtype == torch.float32
+        out.backward(x["grad_out"])
+        assert f.grad.dtype == dt and d.grad.dtype == dt
+        grads[dt] = (out.detach(), f.grad.float(), d.grad.float())
+    eps = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    assert torch.equal(grads[dtype][0], grads[torch.float32][0])          # same inputs, fp32 arithmetic
+    for got, ref in zip(grads[dtype][1:], grads[torch.float32][1:]):
+        assert torch.all((got - ref).abs() <= eps * ref.abs() + 1e-6)     # one rounding to the leaf dtype
+
+
+@pytest.mark.gpu
+def test_module_under_autocast():
+    """With autocast the two heads produce half maps and the operator consumes them directly."""
+    vt, inp, _ = make_module_and_input("laplace", "cuda")
+    with torch.no_grad():
+        ref, _ = vt(inp)
+        with torch.autocast("cuda", dtype=torch.float16):
+            got, depths = vt(inp)
+    assert depths.dtype == torch.float16 and got.dtype == torch.float32
+    m = U.reference_metrics(got.cpu().numpy(), ref.cpu().numpy())
+    assert m["cosine"] > 0.999 and m["mae"] < 1e-3, m
