@@ -73,6 +73,17 @@ def test_validation_status_codes_without_gpu():
     assert capi.backward_gather(ok, 16, 16, 16, 16, 16, 16, 0, 0) == -1            # no workspace
     assert capi.backward_gather(ok, 16, 16, 16, 16, 16, 16, 32, 8) == -2           # workspace too small
     assert capi.sample_geometry(ok, 0, 16, 16, 16) == -1
+    pillar = capi.FbevPillarProblem(channels=8, n_intervals=3, batch=1, num_cams=2, feat_h=4, feat_w=6, epsilon=1e-6,
+                                    depth_distribution=1)
+    ptrs = [16] * 10
+    assert capi.pillarpool_forward(pillar, *([0] + ptrs[1:])) == -1
+    assert capi.pillarpool_forward(pillar, 20, *ptrs[1:]) == -5                      # depth is read as float2
+    pillar.depth_distribution = 2
+    assert capi.pillarpool_forward(pillar, *ptrs) == -3                              # parametric models only
+    pillar.depth_distribution, pillar.channels = 0, 0
+    assert capi.pillarpool_forward(pillar, *ptrs) == -2
+    pillar.channels, pillar.n_intervals = 8, 0
+    assert capi.pillarpool_forward(pillar, *([0] * 10)) == 0                         # nothing to pool
     for rc in range(-6, 1):
         assert capi.status_string(rc) != "unknown status"
     assert capi.status_string(-99) == "unknown status"
