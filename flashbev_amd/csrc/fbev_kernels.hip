@@ -86,7 +86,7 @@ constexpr int kReplicas = 1 << kReplicaBits;
 // block that later gathers it.
 constexpr int kFixedReplicas = 4;
 constexpr int kFixedMinSegment = 16;          // shorter segments would mostly overflow: count instead
-static_assert(kFixedReplicas == kWavesPerBlock, "one fixed segment per wavefront of the texel block");
+static_assert(kFixedReplicas == 4, "the texel pass reads a texel's claim counters as one int4");
 constexpr int kScanChunkBits = 12;           // counters are prefix-summed in chunks of 4096
 
 struct KParams {
@@ -1029,8 +1029,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
 constexpr int kTexelMaxSplit = 8;
 constexpr int kTexelSplitBelow = 8192;
 constexpr int kTexelPart = 128;
-template <int VEC>
-__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_kernel(
+constexpr int kTexelNarrowFrom = 50000;
+constexpr int kTexelNarrowPairs = 2048;      // upper bound of pairs per texel: four per sample
+template <int VEC, int WAVES>
+__global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
     const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
     float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs) {
@@ -1039,8 +1041,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
-    // this wavefront's pairs: [wave_start, wave_end) in steps of wave_stride
-    int wave_start, wave_end, wave_stride;
+    constexpr int n_waves = WAVES, kSegs = kFixedReplicas / WAVES;
+    // this wavefront's pairs: n_segs segments [seg_start[i], seg_end_[i]) walked in steps of wave_stride
+    int seg_start[kSegs], seg_end_[kSegs], n_segs = 0, wave_stride;
     bool shared_texel;
     if (chunk_prefix != nullptr) {
         // counted segments, one after the other: from the end of the previous texel's last
@@ -1052,26 +1055,32 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
         const int n_all = end - start;
         const int n_parts = min((int)gridDim.y, (n_all + kTexelPart - 1) / kTexelPart);
         if ((int)blockIdx.y >= n_parts) return;
-        wave_start = start + (int)(((long long)n_all * blockIdx.y) / n_parts) + wave * kWave;
-        wave_end = start + (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
-        wave_stride = kWavesPerBlock * kWave;
+        seg_start[0] = start + (int)(((long long)n_all * blockIdx.y) / n_parts) + wave * kWave;
+        seg_end_[0] = start + (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
+        n_segs = 1;
+        wave_stride = n_waves * kWave;
         shared_texel = n_parts > 1;
     } else {
-        // fixed segments of pair_cap pairs, one per wavefront; seg_end holds how many were claimed
+        // fixed segments of pair_cap pairs, dealt to the wavefronts in turn; seg_end holds how many were claimed
         const int4 c = *reinterpret_cast<const int4 *>(seg_end + (size_t)t * kFixedReplicas);
         const int n_max = min(max(max(c.x, c.y), max(c.z, c.w)), pair_cap);
         const int n_parts = min((int)gridDim.y, (n_max + kTexelPart - 1) / kTexelPart);
         if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
-        const int mine = min(wave == 0 ? c.x : (wave == 1 ? c.y : (wave == 2 ? c.z : c.w)), pair_cap);
-        const int base = (t * kFixedReplicas + wave) * pair_cap;
-        wave_start = base + (int)(((long long)mine * blockIdx.y) / n_parts);
-        wave_end = base + (int)(((long long)mine * (blockIdx.y + 1)) / n_parts);
+#pragma unroll
+        for (int i = 0; i < kSegs; ++i) {
+            const int r = wave + i * WAVES;          // wavefront w takes segments w, w + WAVES, ...
+            const int mine = min(r == 0 ? c.x : (r == 1 ? c.y : (r == 2 ? c.z : c.w)), pair_cap);
+            const int base = (t * kFixedReplicas + r) * pair_cap;
+            seg_start[i] = base + (int)(((long long)mine * blockIdx.y) / n_parts);
+            seg_end_[i] = base + (int)(((long long)mine * (blockIdx.y + 1)) / n_parts);
+        }
+        n_segs = kSegs;
         wave_stride = kWave;
         shared_texel = n_parts > 1;
     }
     const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
     const int wpw = kWave / lanes_per_row;            // workers per wavefront
-    const int nw = wpw * kWavesPerBlock;
+    const int nw = wpw * n_waves;
     const int wslot = lane / lanes_per_row;
     const int lir = lane - wslot * lanes_per_row;
     const bool worker_lane = wslot < wpw;
@@ -1098,8 +1107,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_texel_ker
         // load, and hands them to its workers through lane shuffles; four grad_out rows per
         // worker are in flight before the first is used.  The loop is bound by load latency:
         // without this the pair load and the row load it addresses form a dependent chain.
-        for (int bstart = wave_start; bstart < wave_end; bstart += wave_stride) {
-            const int nb = min(kWave, wave_end - bstart);
+#pragma unroll
+        for (int sg = 0; sg < kSegs; ++sg)
+        for (int bstart = sg < n_segs ? seg_start[sg] : 0; sg < n_segs && bstart < seg_end_[sg]; bstart += wave_stride) {
+            const int nb = min(kWave, seg_end_[sg] - bstart);
             float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f);
             if (lane < nb) pr = *reinterpret_cast<const float4 *>(pairs + bstart + lane);
             const int word = __float_as_int(pr.x);
@@ -2166,7 +2177,12 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const int vec = vec4 ? 4 : 1;
     const int cq = (p->channels + vec - 1) / vec;
     const int lpr = cq < kWave ? cq : kWave;
-    const int nw = (kWave / lpr) * kWavesPerBlock;
+    // Four wavefronts per texel, or one (taking the four segments in turn) when there are many
+    // texels whose lists cannot be long: measured at 67 584 texels with about 57 pairs each, one
+    // wavefront is 24 % faster than four; at 33 792 texels with about 280 pairs, two are 18 % slower.
+    const bool short_lists = texels >= kTexelNarrowFrom && fbev_backward_max_pairs(p) / (uint64_t)texels < kTexelNarrowPairs;
+    const int texel_waves = short_lists ? 1 : kWavesPerBlock;
+    const int nw = (kWave / lpr) * texel_waves;
     // the depth gradient rides on the pairs exactly when the cell pass folds it in (one channel pass
     // and room for the depth bin in a pair's first word)
     const int from_pairs =
@@ -2176,12 +2192,19 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     long long want_split = kTexelSplitBelow / texels;
     const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);
-    if (vec4)
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<4>), dim3((unsigned)texels, n_split), dim3(kWave * kWavesPerBlock), lds,
-                           st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
+    const dim3 tgrid((unsigned)texels, n_split), tblock(kWave * texel_waves);
+    if (vec4 && short_lists)
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<4, 1>), tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor,
+                           pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
+    else if (vec4)
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<4, kWavesPerBlock>), tgrid, tblock, lds, st, pl.k, grad_out,
+                           prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
+    else if (short_lists)
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<1, 1>), tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor,
+                           pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
     else
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<1>), dim3((unsigned)texels, n_split), dim3(kWave * kWavesPerBlock), lds,
-                           st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
+        hipLaunchKernelGGL((fbev_backward_texel_kernel<1, kWavesPerBlock>), tgrid, tblock, lds, st, pl.k, grad_out,
+                           prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
