@@ -280,3 +280,22 @@ def test_workspace_limit_selects_the_packed_layout(monkeypatch):
     monkeypatch.setenv("FLASHBEV_WORKSPACE_MB", "16")
     assert op_module._pair_capacity(1, 6, [128, 128, 8]) == 16 * 2 ** 20 // 16       # 50 MB would be needed
     assert op_module._pair_capacity(1, 1, [32, 32, 4]) == -1
+
+
+def test_difference_harness_metrics_and_verdict():
+    """flashbev_amd.profile_differences keeps the reference's metric keys, thresholds and
+    pass/fail record (tools/profile_differences.py:17-127)."""
+    from flashbev_amd import profile_differences as pd
+
+    a = torch.tensor([1.0, -2.0, 4.0, 0.0])
+    same = pd.compare_two_methods(a, a.clone(), "A", "B")
+    assert same["overall_match"] and same["metrics"]["mse"] == 0.0 and same["metrics"]["cosine_similarity"] == pytest.approx(1.0)
+    assert set(same["metrics"]) == {"mse", "mae", "max_abs_diff", "min_abs_diff", "mean_diff", "std_diff",
+                                    "max_relative_error", "mean_relative_error", "cosine_similarity"}
+    off = pd.compare_two_methods(a, a + torch.tensor([0.0, 0.0, 0.4, 0.0]), "A", "B")
+    assert off["metrics"]["mse"] == pytest.approx(0.04) and off["metrics"]["mae"] == pytest.approx(0.1)
+    assert off["metrics"]["max_relative_error"] == pytest.approx(0.1) and not off["overall_match"]
+    assert off["pass_fail"] == {"mse": False, "mae": False, "mean_relative_error": False, "cosine_similarity": False}
+    assert "error" in pd.compare_two_methods(a, a[:2])
+    zero = pd.compute_difference_metrics(torch.zeros(3), torch.zeros(3))
+    assert zero["cosine_similarity"] == 1.0
