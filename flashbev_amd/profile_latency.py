@@ -31,7 +31,7 @@ import numpy as np
 import torch
 
 from .flash_bevpool import flash_bevpool
-from .rig import rig_projection, surround_rig
+from .rig import load_calibration_params, rig_projection, surround_rig
 from .sampling_vt import SamplingVT
 from .workloads import SURROUND_YAWS
 
@@ -69,6 +69,9 @@ def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
     ap.add_argument("--backward", action="store_true")
     ap.add_argument("--with-baseline", action="store_true",
                     help="module mode: also time the Sampling-VT+PillarPool method (forward only)")
+    ap.add_argument("--load-calib", default=None,
+                    help="calibration JSON in the reference's layout (inputs/calib_nuscenes.json) instead of the "
+                         "synthetic surround rig; cameras are taken from it in order")
     ap.add_argument("--device", default="cuda")
     ap.add_argument("--output-json", default=None)
     return ap.parse_args(argv)
@@ -129,6 +132,12 @@ def run_point(args: argparse.Namespace, num_bins: int, num_cams: int, threshold:
     yaws = tuple(SURROUND_YAWS[i % len(SURROUND_YAWS)] for i in range(num_cams))
     fx = 560.0 * args.input_w / 704.0
     rig = surround_rig(B, yaws, fx, fx, args.input_w / 2.0, args.input_h / 2.0, seed=args.seed)
+    if args.load_calib:
+        calib = load_calibration_params(args.load_calib)
+        if calib["camera2imgs"].shape[1] < num_cams:
+            raise ValueError(f"{args.load_calib} holds {calib['camera2imgs'].shape[1]} cameras, {num_cams} asked for")
+        rig = {k: (v[:1].expand(B, *v.shape[1:]) if k == "bda" else v[:1, :num_cams].expand(B, num_cams, *v.shape[2:])
+                   ).contiguous() for k, v in calib.items()}
     g = torch.Generator().manual_seed(args.seed)
     dist = 1 if args.depth_distribution == "laplace" else 0
     base = {"method": METHOD, "num_height_bins": num_bins, "num_cameras": num_cams, "z_resolution": grid["z"][2],

@@ -32,6 +32,21 @@ def create_projection_matrix(sensor2ego, ego2global, camera2imgs, post_rots, pos
     return torch.matmul(intrinsic, ego2sensor)[:, :, :3, :].contiguous()
 
 
+def load_calibration_params(input_path: str, device: str = "cpu") -> dict:
+    """Calibration tensors from a JSON file in the reference's layout
+    (tools/utils/data_utils.py:9-24; inputs/calib_nuscenes.json): sensor2ego, ego2global [B,N,4,4],
+    camera2imgs, post_rots [B,N,3,3], post_trans [B,N,3], bda [B,4,4], float32."""
+    import json
+
+    with open(input_path, "r") as fh:
+        raw = json.load(fh)
+    keys = ("sensor2ego", "ego2global", "camera2imgs", "post_rots", "post_trans", "bda")
+    missing = [k for k in keys if k not in raw]
+    if missing:
+        raise KeyError(f"{input_path}: calibration file lacks {missing}")
+    return {k: torch.tensor(raw[k], dtype=torch.float32, device=device) for k in keys}
+
+
 def _rot(axis: str, a: float) -> np.ndarray:
     c, s = math.cos(a), math.sin(a)
     if axis == "x":

@@ -232,3 +232,25 @@ def test_fixed_segments_overflow_falls_back_to_atomics(dist):
     seg_cap = capi.backward_max_pairs(p) // (w.feat_hw[0] * w.feat_hw[1] * 4)
     assert seg_cap >= 16 and per_texel.max() > 8 * seg_cap, (seg_cap, per_texel.max())
     check_all(w, x, dist, thr=0.0, modes=("gather", "gather_overwrite", "gather_counted"))
+
+
+def test_the_reference_calibration_fixture():
+    """The reference's own six-camera nuScenes calibration (its inputs/calib_nuscenes.json, kept as
+    data under tests/golden/): masks, indices and fractions bit for bit, values within tolerance,
+    with the reference benchmark's grid (tools/config/config.yaml: z in [-4, 2] m, 12 bins)."""
+    import os
+
+    from flashbev_amd.rig import load_calibration_params, rig_projection
+
+    rig = load_calibration_params(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                               "calib_nuscenes.json"))
+    w = small(channels=32, roi_range=(-50.0, 50.0, -50.0, 50.0, -4.0, 2.0), grid_size=(100, 100, 12))
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    x["projection_matrices"] = rig_projection(rig).cuda()
+    mask, idx, frac = U.capi_geometry(x["projection_matrices"], w)
+    ref = c_oracle.geometry(x["projection_matrices"].cpu().numpy(), w.feat_hw, w.image_hw, w.roi_range, w.grid_size)
+    assert 0.05 < ref["mask"].mean() < 0.5
+    assert np.array_equal(mask.cpu().numpy(), ref["mask"]) and np.array_equal(idx.cpu().numpy(), ref["idx"])
+    assert np.array_equal(frac.cpu().numpy().view(np.uint32), ref["frac"].view(np.uint32))
+    check_all(w, x, 1, thr=0.0)
+    check_all(w, x, 0, thr=1e-6, modes=("gather",))

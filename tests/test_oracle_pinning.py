@@ -334,3 +334,31 @@ def test_oracle_reproduces_the_committed_vectors(name):
     assert np.array_equal(got["frac"].view(np.uint32), want["frac"].view(np.uint32))
     for key in ("out", "d_depth", "d_feats"):
         assert np.allclose(got[key], want[key], rtol=1e-6, atol=1e-7), key
+
+
+def test_projection_matrices_of_the_reference_calibration_fixture():
+    """create_projection_matrix on the reference's nuScenes calibration (its
+    inputs/calib_nuscenes.json, kept as data under tests/golden/) against the closed form in
+    float64, and against what such a rig must look like: every camera sees a point 20 m along its
+    optical axis at the image centre, the post-augmentation image being 704x256."""
+    import os
+
+    from flashbev_amd.rig import create_projection_matrix, load_calibration_params
+
+    rig = load_calibration_params(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                               "calib_nuscenes.json"))
+    assert rig["sensor2ego"].shape == (1, 6, 4, 4) and rig["camera2imgs"].shape == (1, 6, 3, 3)
+    P = create_projection_matrix(*[rig[k] for k in ("sensor2ego", "ego2global", "camera2imgs", "post_rots",
+                                                     "post_trans", "bda")]).numpy()
+    assert P.shape == (1, 6, 3, 4)
+    s2e = rig["sensor2ego"].double().numpy()
+    for n in range(6):
+        K = rig["post_rots"][0, n].double().numpy() @ rig["camera2imgs"][0, n].double().numpy()
+        K[:, 2] += rig["post_trans"][0, n].double().numpy()
+        want = (np.hstack([K, np.zeros((3, 1))]) @ np.linalg.inv(s2e[0, n]))
+        assert np.allclose(P[0, n], want, rtol=1e-4, atol=1e-3), n
+        # a point 20 m down the optical axis (camera z) lands at the principal point of the resized image
+        point = s2e[0, n] @ np.array([0.0, 0.0, 20.0, 1.0])
+        u, v, d = P[0, n].astype(np.float64) @ point
+        assert abs(d - 20.0) < 1e-3 and abs(u / d - K[0, 2]) < 0.05 and abs(v / d - K[1, 2]) < 0.05
+        assert 300 < K[0, 2] < 400 and 40 < K[1, 2] < 100          # principal point inside 704x256
