@@ -161,6 +161,37 @@ def time_graph_steps(r: Runner, steps: int, warmup: int):
     return (t1 - t0) * 1e3 / steps
 
 
+def time_operator_steps(r: Runner, steps: int, warmup: int):
+    """The autograd operator as a model calls it: every step allocates its output and gradient
+    buffers and runs through the autograd engine.  Wall-clock ms per forward-only and per
+    forward+backward step; reported beside the pre-allocated figure, never as `value`."""
+    from flashbev_amd import flash_bevpool
+    x, w = r.x, r.w
+    kw = dict(projection_matrices=x["projection_matrices"], feature_size=x["feature_size"],
+              image_size=list(w.image_hw), roi_range=list(w.roi_range), grid_size=list(w.grid_size),
+              depth_distribution=r.dist, epsilon=r.eps, depth_weight_threshold=r.thr, depth_range=w.depth_range)
+    feats = x["image_feats"].clone().requires_grad_(True)
+    depth = x["depth_params"].clone().requires_grad_(True)
+    got = {}
+    for name in ("fwd", "fwd_bwd"):
+        def step():
+            if name == "fwd":
+                with torch.no_grad():
+                    flash_bevpool(image_feats=feats, depth_params=depth, **kw)
+            else:
+                feats.grad = depth.grad = None
+                flash_bevpool(image_feats=feats, depth_params=depth, **kw).backward(x["grad_out"])
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        got[name] = (time.perf_counter() - t0) * 1e3 / steps
+    return got
+
+
 def profile_steps(r: Runner, steps: int):
     """The same steps again with the library's per-kernel event timing switched on."""
     capi.profile_enable(True)
@@ -283,6 +314,7 @@ def main():
     graph_ms = None if args.no_graph else time_graph_steps(r, args.steps, args.warmup)
     ms = eager_ms
     kernels = profile_steps(r, args.steps)
+    op_ms = time_operator_steps(r, args.steps, args.warmup)
     fwd_ms, bwd_ms = statistics.mean(fwd), statistics.mean(bwd)
     kept = int(r.counts.sum().item())          # samples that passed the view and weight tests
     es = 4 if w.dtype == torch.float32 else 2
@@ -309,6 +341,8 @@ def main():
                    "submission": "eager launches on one stream"},
         "ms_per_step_eager": eager_ms, "ms_per_step_graph": graph_ms,
         "fwd_call_ms": stats(fwd), "bwd_call_ms": stats(bwd),
+        # the same work through the autograd operator, output and gradient allocation included
+        "operator_ms_incl_alloc": {"fwd": op_ms["fwd"], "fwd_bwd": op_ms["fwd_bwd"]},
         # not HBM traffic: what the gathers request from the caches (every kept sample reads four
         # feature rows and eight depth values forward, and the same rows plus its cell's
         # grad_out row backward) -- the figure a latency/L2-bound pass is better judged by
