@@ -17,7 +17,7 @@ FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
 EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_columns",
            "fbev_backward_columns_workspace_bytes", "fbev_backward_max_pairs",
-           "fbev_backward_workspace_bytes", "fbev_pillarpool_forward", "fbev_sample_geometry", "fbev_algorithmic_bytes",
+           "fbev_backward_workspace_bytes", "fbev_pillarpool_forward", "fbev_projection_matrices", "fbev_sample_geometry", "fbev_algorithmic_bytes",
            "fbev_profile_enable", "fbev_profile_kernel_count", "fbev_profile_kernel_name",
            "fbev_profile_collect", "fbev_status_string", "fbev_abi_version", "fbev_problem_size")
 
@@ -68,6 +68,8 @@ def load() -> ctypes.CDLL:
         lib.fbev_backward_workspace_bytes.restype = ctypes.c_size_t
         lib.fbev_pillarpool_forward.argtypes = [ctypes.POINTER(FbevPillarProblem)] + [vp] * 11
         lib.fbev_pillarpool_forward.restype = ctypes.c_int
+        lib.fbev_projection_matrices.argtypes = [vp, vp, vp, vp, vp, ctypes.c_int32, vp]
+        lib.fbev_projection_matrices.restype = ctypes.c_int
         lib.fbev_sample_geometry.argtypes = [pp, vp, vp, vp, vp, vp]
         lib.fbev_sample_geometry.restype = ctypes.c_int
         lib.fbev_algorithmic_bytes.argtypes = [pp, ctypes.c_int]
@@ -173,6 +175,12 @@ def pillarpool_forward(p: FbevPillarProblem, depth_ptr, feats_ptr, u_ptr, v_ptr,
     return load().fbev_pillarpool_forward(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(u_ptr), _p(v_ptr),
                                           _p(z_ptr), _p(batch_camera_ptr), _p(ranks_ptr), _p(starts_ptr),
                                           _p(lengths_ptr), _p(out_ptr), _p(stream))
+
+
+def projection_matrices(sensor2ego_ptr: int, camera2imgs_ptr: int, post_rots_ptr: int, post_trans_ptr: int,
+                        proj_ptr: int, count: int, stream: int = 0) -> int:
+    return load().fbev_projection_matrices(_p(sensor2ego_ptr), _p(camera2imgs_ptr), _p(post_rots_ptr),
+                                           _p(post_trans_ptr), _p(proj_ptr), int(count), _p(stream))
 
 
 def sample_geometry(p: FbevProblem, proj_ptr: int, mask_ptr: Optional[int], idx_ptr: Optional[int],

@@ -39,13 +39,13 @@ namespace {
 // call count per kernel.  Disabled (the default) it costs one relaxed atomic load per launch.
 namespace prof {
 enum Kid { kForward, kBackwardScatter, kZero, kCount, kScanChunks, kScanSums, kBackwardCells, kBackwardTexel,
-           kGeometry, kBackwardColumn, kCellCount, kPillar, kNum };
+           kGeometry, kBackwardColumn, kCellCount, kPillar, kProjection, kNum };
 const char *const kNames[kNum] = {"fbev_forward_kernel", "fbev_backward_cells_kernel<scatter>",
                                   "fbev_fill_zero_kernel", "fbev_count_kernel", "fbev_scan_chunks_kernel",
                                   "fbev_scan_sums_kernel", "fbev_backward_cells_kernel<fill>",
                                   "fbev_backward_texel_kernel", "fbev_geometry_kernel",
                                   "fbev_backward_column_kernel", "fbev_forward_kernel<count only>",
-                                  "fbev_pillar_kernel"};
+                                  "fbev_pillar_kernel", "fbev_projection_kernel"};
 struct Rec { hipEvent_t a, b; int kid; };
 std::atomic<bool> enabled{false};
 std::mutex mu;
@@ -1746,6 +1746,49 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_pillar_kernel(
     }
 }
 
+// Projection matrices from calibration, one thread per camera (flashbev/flashbevpool/sampling_vt.py:21-33):
+// K = post_rots * camera2imgs with post_trans added to its third column, E = inverse(sensor2ego),
+// P = rows 0..2 of [K 0; 0 1] * E.  Everything is evaluated in double and rounded once; the inverse is
+// the adjugate over the determinant from 2x2 minors, so a singular sensor2ego gives non-finite
+// entries rather than an error.
+__global__ __launch_bounds__(64) void fbev_projection_kernel(int count, const float *__restrict__ sensor2ego,
+                                                            const float *__restrict__ camera2imgs,
+                                                            const float *__restrict__ post_rots,
+                                                            const float *__restrict__ post_trans,
+                                                            float *__restrict__ proj) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    double a[16], r[9], c[9], kk[9];
+    for (int j = 0; j < 16; ++j) a[j] = (double)sensor2ego[(size_t)i * 16 + j];
+    for (int j = 0; j < 9; ++j) { r[j] = (double)post_rots[(size_t)i * 9 + j]; c[j] = (double)camera2imgs[(size_t)i * 9 + j]; }
+    for (int row = 0; row < 3; ++row)
+        for (int col = 0; col < 3; ++col)
+            kk[row * 3 + col] = (r[row * 3] * c[col] + r[row * 3 + 1] * c[3 + col]) + r[row * 3 + 2] * c[6 + col];
+    for (int row = 0; row < 3; ++row) kk[row * 3 + 2] += (double)post_trans[(size_t)i * 3 + row];
+    const double s0 = a[0] * a[5] - a[4] * a[1], s1 = a[0] * a[6] - a[4] * a[2], s2 = a[0] * a[7] - a[4] * a[3];
+    const double s3 = a[1] * a[6] - a[5] * a[2], s4 = a[1] * a[7] - a[5] * a[3], s5 = a[2] * a[7] - a[6] * a[3];
+    const double c5 = a[10] * a[15] - a[14] * a[11], c4 = a[9] * a[15] - a[13] * a[11], c3 = a[9] * a[14] - a[13] * a[10];
+    const double c2 = a[8] * a[15] - a[12] * a[11], c1 = a[8] * a[14] - a[12] * a[10], c0 = a[8] * a[13] - a[12] * a[9];
+    const double inv_det = 1.0 / (s0 * c5 - s1 * c4 + s2 * c3 + s3 * c2 - s4 * c1 + s5 * c0);
+    double e[12];   // rows 0..2 of the inverse (row 3 only meets the zero column of [K 0; 0 1])
+    e[0] = (a[5] * c5 - a[6] * c4 + a[7] * c3) * inv_det;
+    e[1] = (-a[1] * c5 + a[2] * c4 - a[3] * c3) * inv_det;
+    e[2] = (a[13] * s5 - a[14] * s4 + a[15] * s3) * inv_det;
+    e[3] = (-a[9] * s5 + a[10] * s4 - a[11] * s3) * inv_det;
+    e[4] = (-a[4] * c5 + a[6] * c2 - a[7] * c1) * inv_det;
+    e[5] = (a[0] * c5 - a[2] * c2 + a[3] * c1) * inv_det;
+    e[6] = (-a[12] * s5 + a[14] * s2 - a[15] * s1) * inv_det;
+    e[7] = (a[8] * s5 - a[10] * s2 + a[11] * s1) * inv_det;
+    e[8] = (a[4] * c4 - a[5] * c2 + a[7] * c0) * inv_det;
+    e[9] = (-a[0] * c4 + a[1] * c2 - a[3] * c0) * inv_det;
+    e[10] = (a[12] * s4 - a[13] * s2 + a[15] * s0) * inv_det;
+    e[11] = (-a[8] * s4 + a[9] * s2 - a[11] * s0) * inv_det;
+    for (int row = 0; row < 3; ++row)
+        for (int col = 0; col < 4; ++col)
+            proj[(size_t)i * 12 + row * 4 + col] =
+                (float)((kk[row * 3] * e[col] + kk[row * 3 + 1] * e[4 + col]) + kk[row * 3 + 2] * e[8 + col]);
+}
+
 // ---------------------------------------------------------------- geometry inspection
 __global__ __launch_bounds__(256) void fbev_geometry_kernel(KParams k, const float *__restrict__ proj,
                                                             uint8_t *mask, int32_t *idx, float *frac,
@@ -2272,6 +2315,21 @@ int fbev_sample_geometry(const fbev_problem *p, const float *proj, uint8_t *mask
     prof::Scope timer(prof::kGeometry, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(fbev_geometry_kernel, dim3((unsigned)blocks), dim3(256), 0,
                        static_cast<hipStream_t>(stream), pl.k, proj, mask, idx, frac, total);
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+int fbev_projection_matrices(const float *sensor2ego, const float *camera2imgs, const float *post_rots,
+                             const float *post_trans, float *proj, int32_t count, void *stream) {
+    if (count < 0) return FBEV_ERR_SHAPE;
+    if (count == 0) return FBEV_OK;
+    if (!sensor2ego || !camera2imgs || !post_rots || !post_trans || !proj) return FBEV_ERR_NULL;
+    if ((uintptr_t)sensor2ego % 4 || (uintptr_t)camera2imgs % 4 || (uintptr_t)post_rots % 4 || (uintptr_t)post_trans % 4 ||
+        (uintptr_t)proj % 4)
+        return FBEV_ERR_ALIGNMENT;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    prof::Scope timer(prof::kProjection, st);
+    hipLaunchKernelGGL(fbev_projection_kernel, dim3((unsigned)((count + 63) / 64)), dim3(64), 0, st, (int)count,
+                       sensor2ego, camera2imgs, post_rots, post_trans, proj);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 

@@ -300,6 +300,31 @@ std::vector<at::Tensor> sample_geometry(const at::Tensor &projection_matrices, i
     return {mask, idx, frac};
 }
 
+// create_projection_matrix of the reference's module (flashbev/flashbevpool/sampling_vt.py:21-33) as one launch.
+at::Tensor create_projection_matrix(const at::Tensor &sensor2ego, const at::Tensor &camera2imgs,
+                                    const at::Tensor &post_rots, const at::Tensor &post_trans) {
+    TORCH_CHECK(camera2imgs.is_cuda() && camera2imgs.dim() == 4 && camera2imgs.size(2) == 3 && camera2imgs.size(3) == 3,
+                "create_projection_matrix: camera2imgs must be a GPU tensor [B,N,3,3], got ", camera2imgs.sizes());
+    const int64_t B = camera2imgs.size(0), N = camera2imgs.size(1);
+    TORCH_CHECK(sensor2ego.sizes() == at::IntArrayRef({B, N, 4, 4}), "create_projection_matrix: sensor2ego must be [B,N,4,4], got ",
+                sensor2ego.sizes());
+    TORCH_CHECK(post_rots.sizes() == at::IntArrayRef({B, N, 3, 3}), "create_projection_matrix: post_rots must be [B,N,3,3], got ",
+                post_rots.sizes());
+    TORCH_CHECK(post_trans.sizes() == at::IntArrayRef({B, N, 3}), "create_projection_matrix: post_trans must be [B,N,3], got ",
+                post_trans.sizes());
+    for (const at::Tensor *t : {&sensor2ego, &post_rots, &post_trans}) check_dev(*t, camera2imgs, "a calibration tensor");
+    TORCH_CHECK(B * N < (1ll << 31), "create_projection_matrix: too many cameras");
+    auto f32 = [](const at::Tensor &t) { return t.to(at::kFloat).contiguous(); };
+    const at::Tensor e = f32(sensor2ego), k = f32(camera2imgs), r = f32(post_rots), t = f32(post_trans);
+    at::Tensor proj = at::empty({B, N, 3, 4}, camera2imgs.options().dtype(at::kFloat));
+    DeviceScope scope(camera2imgs.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(camera2imgs.get_device()).stream();
+    raise_on(fbev_projection_matrices(e.data_ptr<float>(), k.data_ptr<float>(), r.data_ptr<float>(), t.data_ptr<float>(),
+                                      proj.data_ptr<float>(), (int32_t)(B * N), st),
+             "fbev_projection_matrices");
+    return proj;
+}
+
 // Same positional order as the reference's sampling_vt_pillarpool_fused_forward
 // (flashbev/flashbevpool/src/sampling_vt.cpp:13-52): note interval_lengths before
 // interval_starts.  All tensors on one device, contiguous; float32 / int32 as in the reference.
@@ -369,5 +394,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);
     m.def("sampling_vt_pillarpool_fused_forward", &sampling_vt_pillarpool_fused_forward,
           "interval pooling over precomputed sample lists (the reference's PillarPool baseline)");
+    m.def("create_projection_matrix", &create_projection_matrix,
+          "[B,N,3,4] projection matrices from sensor2ego, camera2imgs, post_rots, post_trans", py::arg("sensor2ego"),
+          py::arg("camera2imgs"), py::arg("post_rots"), py::arg("post_trans"));
     m.def("abi_version", []() { return fbev_abi_version(); });
 }

@@ -23,6 +23,7 @@ results in the reference either.
 """
 from __future__ import annotations
 
+import functools
 import os
 import weakref
 from typing import Sequence
@@ -94,6 +95,20 @@ def voxel_geometry(roi_range: Sequence[float], grid_size: Sequence[int]):
     return [float(v) for v in r[0::2]], [float(v) for v in size]
 
 
+@functools.lru_cache(maxsize=64)
+def _host_arguments(grid: tuple, image: tuple, roi: tuple):
+    """The small host tensors and voxel geometry of one configuration, built once (they are only
+    read afterwards, by the extension and by the backward)."""
+    vmin, vsize = voxel_geometry(roi, grid)
+    return (torch.tensor(image, dtype=torch.int32), torch.tensor(grid, dtype=torch.int32),
+            torch.tensor(roi, dtype=torch.float32), vmin, vsize)
+
+
+@functools.lru_cache(maxsize=64)
+def _feature_size_table(cameras: int, H: int, W: int):
+    return torch.tensor([H, W], dtype=torch.int32).repeat(cameras)
+
+
 class FlashBEVPool(torch.autograd.Function):
     """Fused projection + depth weighting + bilinear sampling + reduction over cameras and
     height bins.  Returns BEV features [B, Y, X, C] in float32."""
@@ -124,20 +139,17 @@ class FlashBEVPool(torch.autograd.Function):
         d_min, d_step = (1.0, 1.0) if depth_range is None else (float(depth_range[0]), float(depth_range[1]))
 
         B, N, H, W, C = image_feats.shape
-        grid = [int(v) for v in _host_values(grid_size, 3, "grid_size")]
-        image = [int(v) for v in _host_values(image_size, 2, "image_size")]
-        roi = [float(v) for v in _host_values(roi_range, 6, "roi_range")]
-        vmin, vsize = voxel_geometry(roi, grid)
+        grid = tuple(int(v) for v in _host_values(grid_size, 3, "grid_size"))
+        image = tuple(int(v) for v in _host_values(image_size, 2, "image_size"))
+        roi = tuple(float(v) for v in _host_values(roi_range, 6, "roi_range"))
+        image_t, grid_t, roi_t, vmin, vsize = _host_arguments(grid, image, roi)
 
         # feature_size repeats the feature tensor's (H, W) per camera; hand the extension a
         # host copy built from the shape unless the caller already gave a host tensor.
         if isinstance(feature_size, torch.Tensor) and feature_size.device.type == "cpu":
             fs_host = feature_size.to(torch.int32).contiguous()
         else:
-            fs_host = torch.tensor([H, W], dtype=torch.int32).repeat(B * N)
-        image_t = torch.tensor(image, dtype=torch.int32)
-        grid_t = torch.tensor(grid, dtype=torch.int32)
-        roi_t = torch.tensor(roi, dtype=torch.float32)
+            fs_host = _feature_size_table(B * N, H, W)
 
         out = torch.empty((B, grid[1], grid[0], C), dtype=torch.float32, device=image_feats.device)
         red = 0 if reduction == "mean" else 1

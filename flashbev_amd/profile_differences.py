@@ -3,12 +3,13 @@ record layout of the reference's harness (tools/profile_differences.py:17-127).
 
     python -m flashbev_amd.profile_differences [--num-height-bins 12] [--output-json diff.json]
 
-Compares the fused operator (``SamplingVT(fuse_projection=True)``, "FlashBEV(ours)") with the
-baseline method that projects and sorts in PyTorch and pools sample lists
-(``fuse_projection=False, use_bev_pool=True``, "Sampling-VT+PillarPool") on the same seeded
-input and weights.  The reference compares against its dense PyTorch method, which this package
-does not carry; the acceptance thresholds are the reference's (MSE < 1e-6, MAE < 1e-6, mean
-relative error < 1e-3, cosine similarity > 0.9999).
+Builds the reference's three methods with the same seeded weights and input and compares each
+with the first, as tools/profile_differences.py:183-280 does with the method list of
+tools/config/config.yaml:48-60: "Dense PyTorch Sampling-VT" (``fuse_projection=False,
+use_bev_pool=False``, the baseline), "Sampling-VT+PillarPool" (projection and sorting in PyTorch,
+interval pooling kernel) and "FlashBEV(ours)" (the fused operator).  The acceptance thresholds are
+the reference's (MSE < 1e-6, MAE < 1e-6, mean relative error < 1e-3, cosine similarity > 0.9999);
+the JSON file has its layout (:317-340) plus the pass/fail record per method.
 """
 from __future__ import annotations
 
@@ -22,6 +23,11 @@ from .rig import surround_rig
 from .sampling_vt import SamplingVT
 from .workloads import SURROUND_YAWS
 
+METHODS = [
+    {"name": "Dense PyTorch Sampling-VT", "fuse_projection": False, "use_bev_pool": False},
+    {"name": "Sampling-VT+PillarPool", "fuse_projection": False, "use_bev_pool": True},
+    {"name": "FlashBEV(ours)", "fuse_projection": True, "use_bev_pool": False},
+]
 TOLERANCES = {"mse": 1e-6, "mae": 1e-6, "mean_relative_error": 1e-3, "cosine_similarity": 0.9999}
 
 
@@ -95,35 +101,50 @@ def run(args: argparse.Namespace) -> Dict:
            [x] + [rig[k] for k in ("sensor2ego", "ego2global", "camera2imgs", "post_rots", "post_trans", "bda")]]
     kw = dict(grid_config=grid, input_size=(args.input_h, args.input_w), in_channels=args.in_channels,
               out_channels=args.out_channels, depth_distribution=args.depth_distribution, depth_weight_threshold=0.0)
-    torch.manual_seed(args.seed)
-    fused = SamplingVT(**kw).to(args.device).eval()
-    with torch.no_grad():
-        fused.depth_network[0].bias.copy_(torch.tensor([12.0, 1.5]))      # useful means and sigmas from random weights
-    lists = SamplingVT(fuse_projection=False, use_bev_pool=True, **kw).to(args.device).eval()
-    lists.load_state_dict(fused.state_dict(), strict=False)
-    with torch.no_grad():
-        a, _ = fused(inp)
-        b, _ = lists(inp)
-    return compare_two_methods(b, a, "Sampling-VT+PillarPool", "FlashBEV(ours)")
+    outputs, weights = {}, None
+    for method in METHODS:
+        torch.manual_seed(args.seed)
+        vt = SamplingVT(fuse_projection=method["fuse_projection"], use_bev_pool=method["use_bev_pool"], **kw)
+        vt = vt.to(args.device).eval()
+        if weights is None:
+            with torch.no_grad():
+                vt.depth_network[0].bias.copy_(torch.tensor([12.0, 1.5]))   # useful means and sigmas from random weights
+            weights = {k: v for k, v in vt.state_dict().items() if "network" in k}
+        vt.load_state_dict(weights, strict=False)
+        with torch.no_grad():
+            outputs[method["name"]] = vt(inp)[0]
+        del vt
+    baseline = METHODS[0]["name"]
+    report = {"baseline": baseline, "methods": {}}
+    for name, out in outputs.items():
+        entry = {"is_baseline": name == baseline, "output_shape": list(out.shape)}
+        if name != baseline:
+            cmp = compare_two_methods(outputs[baseline], out, baseline, name)
+            entry.update({k: cmp[k] for k in cmp if k not in ("method1", "method2")})
+        report["methods"][name] = entry
+    return report
 
 
 def main(argv: Optional[List[str]] = None) -> None:
     args = parse_args(argv)
     if not torch.cuda.is_available():
         raise SystemExit("profile_differences: no GPU visible")
-    cmp = run(args)
-    if "error" in cmp:
-        raise SystemExit(cmp["error"])
-    print(f"Method 1: {cmp['method1']}\nMethod 2: {cmp['method2']}")
-    for key, value in cmp["metrics"].items():
-        tol = cmp["tolerances"].get(key)
-        mark = "" if tol is None else ("  PASS" if cmp["pass_fail"][key] else "  FAIL") + f" (tolerance {tol:g})"
-        print(f"  {key:22s} {value: .6e}{mark}")
-    print("overall match:", cmp["overall_match"])
+    report = run(args)
+    print(f"Baseline: {report['baseline']}")
+    for name, entry in report["methods"].items():
+        if entry["is_baseline"]:
+            continue
+        if "error" in entry:
+            raise SystemExit(f"{name}: {entry['error']}")
+        print(f"{name} against the baseline:")
+        for key, value in entry["metrics"].items():
+            tol = entry["tolerances"].get(key)
+            mark = "" if tol is None else ("  PASS" if entry["pass_fail"][key] else "  FAIL") + f" (tolerance {tol:g})"
+            print(f"  {key:22s} {value: .6e}{mark}")
+        print("  overall match:", entry["overall_match"])
     if args.output_json:
         with open(args.output_json, "w") as fh:
-            json.dump(cmp, fh, indent=2)
-
+            json.dump(report, fh, indent=2)
 
 if __name__ == "__main__":
     main()

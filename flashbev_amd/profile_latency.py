@@ -16,13 +16,14 @@ operator on generated tensors like ``benchmark_flashbevpool_kernel``
 with the host clock, allocation of the output included, as the reference does.  ``--backward``
 adds a forward+backward record per point (the reference never times its backward).
 
-``--module --with-baseline`` adds the reference's "Sampling-VT+PillarPool" method (projection
-and sorting in PyTorch, interval pooling kernel); its dense PyTorch method has no counterpart
-here.
+``--module --with-baseline`` adds the reference's two other methods (tools/config/config.yaml:48-60):
+"Dense PyTorch Sampling-VT" (grid_sample over the whole frustum volume) and
+"Sampling-VT+PillarPool" (projection and sorting in PyTorch, interval pooling kernel).
 """
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import time
 from typing import Dict, List, Optional
@@ -36,7 +37,7 @@ from .sampling_vt import SamplingVT
 from .workloads import SURROUND_YAWS
 
 METHOD = "FlashBEV(ours)"
-BASELINE_METHOD = "Sampling-VT+PillarPool"
+BASELINE_METHODS = {"Dense PyTorch Sampling-VT": False, "Sampling-VT+PillarPool": True}     # name -> use_bev_pool
 
 
 def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
@@ -68,7 +69,7 @@ def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
     mode.add_argument("--module", dest="kernel_only", action="store_false")
     ap.add_argument("--backward", action="store_true")
     ap.add_argument("--with-baseline", action="store_true",
-                    help="module mode: also time the Sampling-VT+PillarPool method (forward only)")
+                    help="module mode: also time the dense PyTorch and Sampling-VT+PillarPool methods (forward only)")
     ap.add_argument("--load-calib", default=None,
                     help="calibration JSON in the reference's layout (inputs/calib_nuscenes.json) instead of the "
                          "synthetic surround rig; cameras are taken from it in order")
@@ -108,6 +109,7 @@ def time_calls(fn, num_warmup: int, num_iterations: int) -> Dict[str, float]:
     for _ in range(num_warmup):
         fn()
     torch.cuda.synchronize()
+    gc.collect()                      # garbage of the previous point is not collected inside a timed call
     torch.cuda.empty_cache()
     torch.cuda.reset_peak_memory_stats()
     latencies = []
@@ -185,18 +187,19 @@ def run_point(args: argparse.Namespace, num_bins: int, num_cams: int, threshold:
                 return vt(inp)
 
         records.append({**base, "pass": "forward", **time_calls(forward, args.num_warmup, args.num_iterations)})
-        if args.with_baseline:
+        for name, use_bev_pool in (BASELINE_METHODS.items() if args.with_baseline else ()):
             other = SamplingVT(grid, (args.input_h, args.input_w), downsample=args.downsample,
                                in_channels=args.in_channels, out_channels=args.out_channels, fuse_projection=False,
-                               use_bev_pool=True, depth_distribution=args.depth_distribution).to(dev).eval()
+                               use_bev_pool=use_bev_pool, depth_distribution=args.depth_distribution,
+                               depth_weight_threshold=threshold).to(dev).eval()
             other.load_state_dict(vt.state_dict(), strict=False)
 
-            def forward_baseline():
+            def forward_other():
                 with torch.no_grad():
                     return other(inp)
 
-            records.append({**base, "method": BASELINE_METHOD, "fuse_projection": False, "use_bev_pool": True,
-                            "pass": "forward", **time_calls(forward_baseline, args.num_warmup, args.num_iterations)})
+            records.append({**base, "method": name, "fuse_projection": False, "use_bev_pool": use_bev_pool,
+                            "pass": "forward", **time_calls(forward_other, args.num_warmup, args.num_iterations)})
             del other
         if args.backward:
             vt.train()

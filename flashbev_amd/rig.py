@@ -1,10 +1,13 @@
-"""Camera rigs and projection matrices (host-side, tiny).
+"""Camera rigs and projection matrices.
 
 ``create_projection_matrix`` restates flashbev/flashbevpool/sampling_vt.py:21-33: the
 3x4 matrix that maps ego coordinates (x, y, z, 1) to (u*d, v*d, d) in image pixels,
 P = [post_rots @ K | post_trans added to column 2] embedded in a 4x4 identity, times
 inv(sensor2ego), rows 0..2.  ``ego2global`` and ``bda`` are accepted and unused, as in the
-reference.
+reference.  Calibration tensors on the GPU go through one kernel of the HIP library (the
+reference's chain of small PyTorch operations costs more time per call than the pooling
+itself at the benchmark sizes); tensors on the host, which is where rigs and test inputs are
+prepared, are combined with PyTorch operations.
 
 ``surround_rig`` builds the synthetic surround-view calibration the benchmark
 configurations use: pinhole cameras at given yaw angles, mounted ``height`` metres high and
@@ -23,6 +26,9 @@ import torch
 
 def create_projection_matrix(sensor2ego, ego2global, camera2imgs, post_rots, post_trans, bda=None):
     """[B,N,3,4] float32 projection matrices from BEVDet-style calibration tensors."""
+    if camera2imgs.device.type == "cuda":
+        from ._native import load_ext
+        return load_ext().create_projection_matrix(sensor2ego, camera2imgs, post_rots, post_trans)
     B, N = camera2imgs.shape[:2]
     dev, dt = camera2imgs.device, camera2imgs.dtype
     intrinsic = torch.eye(4, device=dev, dtype=dt).repeat(B, N, 1, 1)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 2
+#define FBEV_ABI_VERSION 3
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -190,6 +190,18 @@ int fbev_pillarpool_forward(const fbev_pillar_problem *p, const float *depth, co
  */
 int fbev_sample_geometry(const fbev_problem *p, const float *proj, uint8_t *mask, int32_t *idx,
                          float *frac, void *stream);
+
+/*
+ * Projection matrices from calibration tensors, count = B*N cameras:
+ *   sensor2ego [count,4,4], camera2imgs [count,3,3], post_rots [count,3,3], post_trans [count,3]
+ *   -> proj [count,3,4] = rows 0..2 of [post_rots*camera2imgs (+post_trans on column 2), 0; 0, 1] * inverse(sensor2ego)
+ * Evaluated in double and rounded once to float32.  A singular sensor2ego yields non-finite entries
+ * (the reference's torch.inverse raises instead, after a device synchronisation).
+ * Replaces create_projection_matrix, flashbev/flashbevpool/sampling_vt.py:21-33 (about twenty
+ * small PyTorch launches per call there).
+ */
+int fbev_projection_matrices(const float *sensor2ego, const float *camera2imgs, const float *post_rots,
+                             const float *post_trans, float *proj, int32_t count, void *stream);
 
 /* Compulsory bytes moved by one call: every operand tensor once (backward != 0 selects the backward). */
 uint64_t fbev_algorithmic_bytes(const fbev_problem *p, int backward);

@@ -37,8 +37,8 @@ def test_module_state_dict_names_and_buffers():
     assert vt.sample_grid_size.tolist() == [100, 100, 12] and vt.num_depth_bins == 59
     with pytest.raises(ValueError):
         SamplingVT(GRID, (256, 704), depth_distribution="uniform")
-    with pytest.raises(NotImplementedError):
-        SamplingVT(GRID, (256, 704), fuse_projection=False, use_bev_pool=False)
+    assert SamplingVT(GRID, (256, 704), in_channels=8, out_channels=4, fuse_projection=False,
+                      use_bev_pool=False).coords_3d.shape == (100, 100, 12, 3)
     assert SamplingVT(GRID, (256, 704), in_channels=8, out_channels=4, fuse_projection=False).coords_3d.shape == \
         (100, 100, 12, 3)
     # a step that divides the range only up to rounding still yields the intended count
@@ -206,6 +206,36 @@ def test_module_baseline_branch_agrees_with_the_fused_branch():
     assert a.shape == b.shape == (1, 24, 100, 100)
     m = U.reference_metrics(b.cpu().numpy(), a.cpu().numpy())
     assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["mean_rel"] < 1e-3 and m["cosine"] > 0.9999, m
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("depth_distribution,threshold", [("laplace", 0.0), ("gaussian", 0.0), ("laplace", 1e-4)])
+def test_module_dense_branch_agrees_with_the_fused_branch(depth_distribution, threshold):
+    """fuse_projection=False, use_bev_pool=False (the reference's baseline method: grid_sample over
+    the whole frustum volume) against the fused operator with the same weights, forward by the
+    reference's acceptance statistics and the parameter gradients of a training step."""
+    vt, inp, _ = make_module_and_input(depth_distribution, "cuda")
+    vt.depth_weight_threshold = threshold
+    dense = SamplingVT(GRID, (256, 704), downsample=16, in_channels=32, out_channels=24, fuse_projection=False,
+                       use_bev_pool=False, depth_distribution=depth_distribution,
+                       depth_weight_threshold=threshold).to("cuda").eval()
+    dense.load_state_dict(vt.state_dict(), strict=False)
+    with torch.no_grad():
+        a, _ = vt(inp)
+        b, _ = dense(inp)
+    assert a.shape == b.shape == (1, 24, 100, 100)
+    m = U.reference_metrics(b.cpu().numpy(), a.cpu().numpy())
+    assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["mean_rel"] < 1e-3 and m["cosine"] > 0.9999, m
+    g = torch.Generator().manual_seed(5)
+    target = torch.randn(a.shape, generator=g).cuda()
+    grads = []
+    for module in (vt, dense):
+        module.zero_grad(set_to_none=True)
+        (module(inp)[0] * target).sum().backward()
+        grads.append([p.grad.clone() for p in module.parameters()])
+    for ga, gb, (name, _) in zip(*grads, vt.named_parameters()):
+        scale = gb.abs().max().item()
+        assert (ga - gb).abs().max().item() <= 2e-3 * scale + 1e-6, (name, (ga - gb).abs().max().item(), scale)
 
 
 @pytest.mark.gpu

@@ -254,3 +254,51 @@ def test_the_reference_calibration_fixture():
     assert np.array_equal(frac.cpu().numpy().view(np.uint32), ref["frac"].view(np.uint32))
     check_all(w, x, 1, thr=0.0)
     check_all(w, x, 0, thr=1e-6, modes=("gather",))
+
+
+def test_projection_kernel_against_the_closed_form_in_float64():
+    """fbev_projection_matrices through the C ABI: the reference's nuScenes calibration and seeded
+    surround rigs with image augmentation (rotation, scale, shift) against float64 NumPy -- the
+    kernel evaluates in double and rounds once, so the bound is one rounding of the result (and
+    of its cancellation-prone entries relative to the row's largest term)."""
+    import os
+
+    from flashbev_amd import capi
+    from flashbev_amd.rig import create_projection_matrix, load_calibration_params, surround_rig
+
+    rigs = [load_calibration_params(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                                 "calib_nuscenes.json"))]
+    g = torch.Generator().manual_seed(11)
+    for seed in (1, 2):
+        rig = surround_rig(3, (0.0, 55.0, -55.0, 110.0, -110.0, 180.0), 560.0, 540.0, 352.0, 128.0, seed=seed)
+        ang = (torch.rand(3, 6, generator=g) - 0.5) * 0.2
+        scale = 0.9 + 0.2 * torch.rand(3, 6, generator=g)
+        rot = torch.eye(3).repeat(3, 6, 1, 1)
+        rot[..., 0, 0] = scale * torch.cos(ang); rot[..., 0, 1] = -scale * torch.sin(ang)
+        rot[..., 1, 0] = scale * torch.sin(ang); rot[..., 1, 1] = scale * torch.cos(ang)
+        rig["post_rots"] = rot
+        rig["post_trans"] = torch.cat([torch.randn(3, 6, 2, generator=g) * 20.0, torch.zeros(3, 6, 1)], dim=-1)
+        rigs.append(rig)
+    for rig in rigs:
+        dev = {k: rig[k].cuda().contiguous() for k in ("sensor2ego", "camera2imgs", "post_rots", "post_trans")}
+        B, N = dev["camera2imgs"].shape[:2]
+        out = torch.full((B, N, 3, 4), float("nan"), device="cuda")
+        print(f"[case] projection kernel B={B} N={N}", flush=True)
+        capi.check(capi.projection_matrices(dev["sensor2ego"].data_ptr(), dev["camera2imgs"].data_ptr(),
+                                            dev["post_rots"].data_ptr(), dev["post_trans"].data_ptr(),
+                                            out.data_ptr(), B * N, torch.cuda.current_stream().cuda_stream),
+                   "fbev_projection_matrices")
+        torch.cuda.synchronize()
+        K = rig["post_rots"].double().numpy() @ rig["camera2imgs"].double().numpy()
+        K[..., 2] += rig["post_trans"].double().numpy()
+        want = (K @ np.linalg.inv(rig["sensor2ego"].double().numpy())[..., :3, :])
+        got = out.cpu().numpy().astype(np.float64)
+        bound = 2.0 ** -23 * np.abs(want).max(axis=-1, keepdims=True)
+        assert np.all(np.abs(got - want) <= bound), float(np.abs(got - want).max())
+        # the operator-facing function takes the same route for GPU tensors, and agrees with its host path
+        args = [rig[k] for k in ("sensor2ego", "ego2global", "camera2imgs", "post_rots", "post_trans", "bda")]
+        via_module = create_projection_matrix(*[a.cuda() for a in args])
+        assert torch.equal(via_module, out)
+        assert torch.allclose(create_projection_matrix(*args), out.cpu(), rtol=1e-4, atol=1e-3)
+    assert capi.projection_matrices(0, 0, 0, 0, 0, 0) == 0          # nothing to do
+    assert capi.projection_matrices(0, 0, 0, 0, 0, 4) == -1         # NULL pointers

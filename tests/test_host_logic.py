@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in flashbev_hip.h but not exported"
     assert sorted(capi.EXPORTS) == names
-    assert lib.fbev_abi_version() == 2
+    assert lib.fbev_abi_version() == 3
     assert lib.fbev_problem_size() == ctypes.sizeof(capi.FbevProblem)
 
 
@@ -282,7 +282,7 @@ def test_workspace_limit_selects_the_packed_layout(monkeypatch):
     assert op_module._pair_capacity(1, 1, [32, 32, 4]) == -1
 
 
-def test_difference_harness_metrics_and_verdict():
+def test_difference_harness_metrics_and_pass_fail():
     """flashbev_amd.profile_differences keeps the reference's metric keys, thresholds and
     pass/fail record (tools/profile_differences.py:17-127)."""
     from flashbev_amd import profile_differences as pd
@@ -299,3 +299,47 @@ def test_difference_harness_metrics_and_verdict():
     assert "error" in pd.compare_two_methods(a, a[:2])
     zero = pd.compute_difference_metrics(torch.zeros(3), torch.zeros(3))
     assert zero["cosine_similarity"] == 1.0
+
+
+@pytest.mark.parametrize("dist,thr", [(1, 0.0), (1, 1e-6), (0, 1e-6)])
+def test_dense_method_of_the_module_agrees_with_the_c_oracle(dist, thr):
+    """The dense PyTorch method the harnesses use as their baseline (pure torch, so it runs here)
+    against the C restatement of the fused arithmetic on the same inputs."""
+    from flashbev_amd.sampling_vt import project_coords, sampling_vt_pytorch
+    from oracle import c_oracle
+
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    B, N, H, W, C = x["image_feats"].shape
+    gx, gy, gz = w.grid_size
+    lo, hi = w.roi_range[0::2], w.roi_range[1::2]
+    axes = [torch.linspace(a, b, n + 1)[:-1] + (b - a) / n / 2.0 for a, b, n in zip(lo, hi, (gx, gy, gz))]
+    centres = torch.stack(torch.meshgrid(*axes, indexing="ij"), dim=-1)
+    uvd = project_coords(centres.expand(B, N, gx, gy, gz, 3), x["projection_matrices"])
+    assert uvd.shape == (B, N, gx, gy, gz, 3)
+    got = sampling_vt_pytorch(uvd, x["image_feats"].movedim(-1, 2).flatten(0, 1),
+                              x["depth_params"].movedim(-1, 2).flatten(0, 1), B, N, w.image_hw, thr,
+                              "laplace" if dist == 1 else "gaussian")
+    assert got.shape == (B, C, gy, gx)
+    want = c_oracle.forward(x["depth_params"].numpy(), x["image_feats"].numpy(), x["projection_matrices"].numpy(),
+                            image_size=w.image_hw, roi_range=w.roi_range, grid_size=w.grid_size,
+                            depth_distribution=dist, epsilon=1e-6, depth_weight_threshold=thr)
+    close = np.isclose(got.movedim(1, -1).numpy(), want, rtol=1e-3, atol=1e-5).all(axis=-1)
+    assert (~close).sum() <= 2, int((~close).sum())        # a sample within rounding of a border may flip
+
+
+def test_module_selects_the_method_from_its_flags():
+    from flashbev_amd import SamplingVT
+    grid = {"x": [-8.0, 8.0, 1.0], "y": [-8.0, 8.0, 1.0], "z": [-2.0, 2.0, 1.0], "depth": [1.0, 30.0, 1.0]}
+    kw = dict(grid_config=grid, input_size=(64, 176), in_channels=8, out_channels=4)
+    assert SamplingVT(**kw)._method().__name__ == "_pool"
+    assert SamplingVT(fuse_projection=False, use_bev_pool=True, **kw)._method().__name__ == "_pool_sorted_lists"
+    dense = SamplingVT(fuse_projection=False, use_bev_pool=False, **kw)
+    assert dense._method().__name__ == "_pool_dense" and dense.coords_3d.shape == (16, 16, 4, 3)
+
+
+def test_projection_entry_point_validates_without_gpu():
+    assert capi.projection_matrices(0, 0, 0, 0, 0, 0) == 0          # nothing to do
+    assert capi.projection_matrices(0, 0, 0, 0, 0, -1) == -2        # negative count
+    assert capi.projection_matrices(0, 0, 0, 0, 0, 4) == -1         # NULL pointers
+    assert capi.projection_matrices(8, 16, 16, 16, 18, 4) == -5     # misaligned output
