@@ -114,6 +114,7 @@ struct KParams {
     int n_blocks;
     int waves;           // wavefronts per block of the cell-centric kernels
     int bin_bits;        // a pair's first word is cell << bin_bits | depth bin; -1: the word cannot hold both
+    int row_units;       // a texel's feature row in address units: 16 bytes on the vector paths, else one element
 };
 
 // ---------------------------------------------------------------- element access
@@ -351,7 +352,9 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 
 // Entry of a compacted list: ENTRY_F4 float4 words.
 //   forward   word 0: corner weights already multiplied by the depth weight
-//             word 1: four texel indices ((b*N+n)*H + v)*W + u as int bits (t00, t01, t10, t11)
+//             word 1: where the four texels' feature rows start, in address units (texel index
+//                     ((b*N+n)*H + v)*W + u times KParams::row_units) as int bits (t00, t01, t10, t11):
+//                     the gather loop then forms an address with one shift-add, not a 64-bit multiply
 //   backward  word 0: du, dv, t00, (u1 != u0) | (v1 != v0) << 1 -- the four weights and texels
 //                     follow from these exactly as phase A computed them
 //             word 1: wgt, a, b, (k0 | k1 << 16)
@@ -499,8 +502,8 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
             float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
             e[0] = w0;
             e[1] = BACKWARD ? w2
-                            : make_float4(__int_as_float(tx.x), __int_as_float(tx.y), __int_as_float(tx.z),
-                                          __int_as_float(tx.w));
+                            : make_float4(__int_as_float(tx.x * k.row_units), __int_as_float(tx.y * k.row_units),
+                                          __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
         }
         if (MODE == kModeFill && keep) {
             // claim one position per corner in the texel's segment of the pair array; the four
@@ -566,6 +569,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     const int lis = lane - slot * k.lanes_per_slot;
     const bool carrier = slot < k.slots;
     const int span = k.lanes_per_slot * VEC * CPL;   // channels covered per pass
+    constexpr int kUnitShift = VEC > 1 ? 4 : (sizeof(T) == 4 ? 2 : 1);
+    const char *fbytes = reinterpret_cast<const char *>(feats);
 
     for (int r = 0; r < k.rounds; ++r) {
         const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
@@ -587,13 +592,14 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
             for (int j = 0; j < CPL; ++j)
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) acc[j][v] = 0.0f;
-            for (int e = 0; e < n; ++e) {
+            // one entry: four row loads per channel vector, then the weighted sum
+            auto gather = [&](int e) {
                 float4 w = my[2 * e];
                 float4 tf = my[2 * e + 1];
-                const T *p00 = feats + (size_t)__float_as_int(tf.x) * k.C;
-                const T *p01 = feats + (size_t)__float_as_int(tf.y) * k.C;
-                const T *p10 = feats + (size_t)__float_as_int(tf.z) * k.C;
-                const T *p11 = feats + (size_t)__float_as_int(tf.w) * k.C;
+                const T *p00 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.x) << kUnitShift));
+                const T *p01 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.y) << kUnitShift));
+                const T *p10 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.z) << kUnitShift));
+                const T *p11 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.w) << kUnitShift));
 #pragma unroll
                 for (int j = 0; j < CPL; ++j) {
                     int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
@@ -614,7 +620,28 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
                         }
                     }
                 }
+            };
+            // two entries per trip where the registers allow, all eight row loads issued before the
+            // first is used (the loop is a chain of gather latencies, not of arithmetic)
+            int e = 0;
+            if (CPL == 1) {
+                const int ch = c0 + lis * VEC;
+                for (; ch < k.C && e + 1 < n; e += 2) {
+                    const float4 wa = my[2 * e], ta = my[2 * e + 1], wb = my[2 * e + 2], tb = my[2 * e + 3];
+                    const int off[8] = {__float_as_int(ta.x), __float_as_int(ta.y), __float_as_int(ta.z), __float_as_int(ta.w),
+                                        __float_as_int(tb.x), __float_as_int(tb.y), __float_as_int(tb.z), __float_as_int(tb.w)};
+                    const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+                    float f[8][VEC];
+#pragma unroll
+                    for (int c = 0; c < 8; ++c)
+                        VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)off[c] << kUnitShift)) + ch, f[c]);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c)
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[0][v] = __builtin_fmaf(wv[c], f[c][v], acc[0][v]);
+                }
             }
+            for (; e < n; ++e) gather(e);
             if (mine) {
                 const float nf = (float)n;
 #pragma unroll
@@ -818,6 +845,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     // The depth gradient travels with the pairs when one channel pass sees the whole of G and
     // the pair's first word has room for the depth bin; otherwise it is added with atomics here.
     const bool fold = FILL && need_G && k.C <= span && k.bin_bits >= 0;
+    constexpr int kUnitShift = VEC > 1 ? 4 : (sizeof(T) == 4 ? 2 : 1);
+    const char *fbytes = reinterpret_cast<const char *>(feats);
+    const unsigned row_step_v = (unsigned)(k.W * k.row_units);      // one feature-map row down
 
     for (int r = 0; r < k.rounds; ++r) {
         const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
@@ -880,8 +910,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 const float w00 = (1.0f - du) * (1.0f - dv), w01 = (1.0f - du) * dv, w10 = du * (1.0f - dv), w11 = du * dv;
                 const int t00 = __float_as_int(geo.z), fl = __float_as_int(geo.w);
                 const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
-                const size_t o00 = (size_t)t00 * k.C, o01 = (size_t)(t00 + sv) * k.C;
-                const size_t o10 = (size_t)(t00 + su) * k.C, o11 = (size_t)(t00 + sv + su) * k.C;
+                // feature rows in address units: one 32-bit multiply and three adds, then a shift-add each
+                const unsigned r00 = (unsigned)t00 * (unsigned)k.row_units;
+                const unsigned r01 = r00 + ((fl & 2) ? row_step_v : 0u);
+                const unsigned r10 = r00 + ((fl & 1) ? (unsigned)k.row_units : 0u), r11 = r01 + (r10 - r00);
                 bool s00 = true, s01 = true, s10 = true, s11 = true;
                 if (FILL) {
                     const float4 pf = my[EF4 * e + 2];
@@ -895,10 +927,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                     if (ch < k.C) {
                         if (need_G) {
                             float f00[VEC], f01[VEC], f10[VEC], f11[VEC];
-                            VecLoad<T, VEC>::ld(feats + o00 + ch, f00);
-                            VecLoad<T, VEC>::ld(feats + o01 + ch, f01);
-                            VecLoad<T, VEC>::ld(feats + o10 + ch, f10);
-                            VecLoad<T, VEC>::ld(feats + o11 + ch, f11);
+                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r00 << kUnitShift)) + ch, f00);
+                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r01 << kUnitShift)) + ch, f01);
+                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r10 << kUnitShift)) + ch, f10);
+                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r11 << kUnitShift)) + ch, f11);
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) {
                                 const float f = __builtin_fmaf(w11, f11[v], __builtin_fmaf(w10, f10[v],
@@ -907,6 +939,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                             }
                         }
                         if (d_feats != nullptr && (s00 || s01 || s10 || s11)) {
+                            const size_t o00 = (size_t)t00 * k.C, o01 = (size_t)(t00 + sv) * k.C;
+                            const size_t o10 = (size_t)(t00 + su) * k.C, o11 = (size_t)(t00 + sv + su) * k.C;
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) {
                                 if (s00) atomic_add_f32(d_feats + o00 + ch + v, g[j][v] * a00);
@@ -1100,6 +1134,9 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
         for (int i = threadIdx.x; i < k.Dd; i += blockDim.x) bins[i] = 0.0f;
         __syncthreads();
     }
+    constexpr int kOutShift = VEC > 1 ? 4 : 2;
+    const unsigned out_units = (unsigned)(VEC > 1 ? k.C / 4 : k.C);
+    const char *gbytes = reinterpret_cast<const char *>(grad_out);
     for (int c0 = 0; c0 < k.C; c0 += span) {
         const int ch = c0 + lir * VEC;
         const bool on = worker_lane && ch < k.C;
@@ -1123,7 +1160,8 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             // keeps a logic error from turning into a wild read (such a pair counts as cell 0
             // with coefficient 0)
             const bool valid = (unsigned)(word >> bin_bits) < n_cells;
-            const int my_cell = valid ? (word >> bin_bits) : 0;
+            // where the pair's grad_out row starts, in units of 16 bytes (one float off the vector path)
+            const unsigned my_row = valid ? (unsigned)(word >> bin_bits) * out_units : 0u;
             const float my_coef = valid ? pr.y : 0.0f;
             if (c0 == 0 && valid) {
                 if (bin_sums) {
@@ -1146,9 +1184,9 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
 #pragma unroll
                 for (int q = 0; q < UNR; ++q) {
                     const int j = i + q * wpw + wslot_eff;
-                    const int c = __shfl(my_cell, j, kWave);
+                    const unsigned row = (unsigned)__shfl((int)my_row, j, kWave);
                     coefs[q] = __shfl(my_coef, j, kWave);
-                    VecLoad<float, VEC>::ld(grad_out + (size_t)c * k.C + ch_eff, g[q]);
+                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)row << kOutShift)) + ch_eff, g[q]);
                 }
 #pragma unroll
                 for (int q = 0; q < UNR; ++q)
@@ -1157,11 +1195,11 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             }
             for (int i = full; i < nb; i += wpw) {
                 const int j = i + wslot_eff;
-                const int c = __shfl(my_cell, min(j, kWave - 1), kWave);
+                const unsigned row = (unsigned)__shfl((int)my_row, min(j, kWave - 1), kWave);
                 const float coef = __shfl(my_coef, min(j, kWave - 1), kWave);
                 if (j < nb) {
                     float g[VEC];
-                    VecLoad<float, VEC>::ld(grad_out + (size_t)c * k.C + ch_eff, g);
+                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)row << kOutShift)) + ch_eff, g);
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coef, g[v], acc[v]);
                 }
@@ -1886,6 +1924,12 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     const int es = elem_size(p->in_dtype);
     const int full_vec = 16 / es;
     plan->vec = (allow_vec && k.C % full_vec == 0) ? full_vec : 1;
+    {
+        // feature rows are addressed in 32-bit units (16 bytes, or one element off the vector paths)
+        const long long units = plan->vec > 1 ? (long long)k.C * es / 16 : k.C;
+        if ((long long)k.B * k.N * k.H * k.W * units >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+        k.row_units = (int)units;
+    }
     const int cq = (k.C + plan->vec - 1) / plan->vec;      // channel vectors per texel
     int lps = cq < kWave ? cq : kWave;
     int cpl = (cq + lps - 1) / lps;
@@ -2176,6 +2220,10 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
     // pair positions are 32-bit: every sample corner must be countable
     if (4 * sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    // the texel pass addresses grad_out rows in 32-bit units (16 bytes, or one float off the vector path)
+    const bool rows_vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
+    if ((long long)p->batch * p->grid_y * p->grid_x * (rows_vec4 ? p->channels / 4 : p->channels) >= (1ll << 32))
+        return FBEV_ERR_TOO_LARGE;
     size_t cap64 = (workspace_bytes - index_bytes) / sizeof(Pair);
     const int cap = cap64 > 0x7fffffffull ? 0x7fffffff : (int)cap64;
     Plan pl;
