@@ -115,6 +115,7 @@ struct KParams {
     int waves;           // wavefronts per block of the cell-centric kernels
     int bin_bits;        // a pair's first word is cell << bin_bits | depth bin; -1: the word cannot hold both
     int row_units;       // a texel's feature row in address units: 16 bytes on the vector paths, else one element
+    int gz_magic, gz_shift;   // i / gz == (i * gz_magic) >> gz_shift for 0 <= i < 4096
 };
 
 // ---------------------------------------------------------------- element access
@@ -178,14 +179,16 @@ struct Geom {
 
 // One sample in the canonical operation order (each line is one rounded fp32 operation
 // sequence, left to right; no contraction).  P points at 12 floats.
-__device__ __forceinline__ Geom project_sample(const KParams &k, const float *P, float x, float y, float z) {
+// The (x, y) part of the three dot products is shared by all height bins of a (cell, camera)
+// column: au = P[0] * x + P[1] * y, av and ad likewise.
+__device__ __forceinline__ Geom project_column(const KParams &k, const float *P, float au, float av, float ad, float z) {
     Geom g;
     g.valid = false;
     g.u0 = g.u1 = g.v0 = g.v1 = 0;
     g.du = g.dv = 0.0f;
-    float U = ((P[0] * x + P[1] * y) + P[2] * z) + P[3];
-    float V = ((P[4] * x + P[5] * y) + P[6] * z) + P[7];
-    float D = ((P[8] * x + P[9] * y) + P[10] * z) + P[11];
+    float U = (au + P[2] * z) + P[3];
+    float V = (av + P[6] * z) + P[7];
+    float D = (ad + P[10] * z) + P[11];
     g.depth = D;
     if (!(D > 0.0f)) return g;
     float dc = fmaxf(D, k.eps);
@@ -203,6 +206,10 @@ __device__ __forceinline__ Geom project_sample(const KParams &k, const float *P,
     g.v1 = min(max(g.v0 + 1, 0), k.H - 1);
     g.valid = true;
     return g;
+}
+
+__device__ __forceinline__ Geom project_sample(const KParams &k, const float *P, float x, float y, float z) {
+    return project_column(k, P, P[0] * x + P[1] * y, P[4] * x + P[5] * y, P[8] * x + P[9] * y, z);
 }
 
 __device__ __forceinline__ float voxel_coord(float lo, int i, float step) {
@@ -302,9 +309,9 @@ __device__ __forceinline__ unsigned long long lanemask_lt(int lane) {
 __device__ __forceinline__ unsigned long long lanemask_le(int lane) { return ~0ull >> (63 - lane); }
 
 // LDS of one block of the cell-centric kernels (float4 units):
-//   [matrices: N*12 floats][decode table: slots*NZ ints]
-//   per wavefront: [16 ints of list lengths][16 float4 of cell centres][slots*NZ ints of
-//   candidates][slots * list_cap entries]
+//   [matrices: N*12 floats][column table: slots*N ints]
+//   per wavefront: [16 ints of list lengths][16 float4 of cell centres][slots*N column records]
+//   [slots*N ints: columns in view][slots*NZ ints of candidates][slots * list_cap entries]
 // Counters that several lanes of a wavefront update in turn live in LDS and are read as
 // volatile.  The pointer carries the LDS address space: a volatile access through a generic
 // pointer becomes a system-coherent flat load that first waits for every outstanding global
@@ -313,38 +320,42 @@ using lds_counter = volatile __attribute__((address_space(3))) int;
 
 struct WaveLds {
     const float *Pm;
-    const int *dec;       // sample index within the wavefront's round -> slot << 28 | camera << 16 | height bin
+    const int *dec;       // column index within the wavefront's round -> slot << 28 | camera << 16
     lds_counter *cnt;     // entries per slot
     float4 *cell;         // per slot: x, y, valid flag, ix | iy << 16
-    int *cand;            // samples that survive the cheap test
+    float4 *col;          // per column: the (x, y) part of U, V, D, and its dec word
+    int *alive;           // columns with a height bin that may be in view
+    unsigned *cand;       // samples that survive the cheap test: column << 16 | height bin
     float4 *lst;
 };
 
 __device__ __forceinline__ int lds_p_f4(const KParams &k) { return (k.N * 12 + 3) / 4; }
-__device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots * k.NZ + 3) / 4; }
+__device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots * k.N + 3) / 4; }
+__device__ __forceinline__ int lds_cand_f4(const KParams &k) { return (k.slots * k.NZ + 3) / 4; }
 
-// Stage the block's matrices and the decode table; returns the wavefront's view.  Ends with a
+// Stage the block's matrices and the column table; returns the wavefront's view.  Ends with a
 // barrier.
 __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *smem, const float *__restrict__ proj,
                                                    int b, int entry_f4) {
     WaveLds L;
     float *Pm = reinterpret_cast<float *>(smem);
     int *dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
-    const int dec_f4 = lds_dec_f4(k);
-    const int per_wave_f4 = 4 + 16 + dec_f4 + k.slots * k.list_cap * entry_f4;
+    const int dec_f4 = lds_dec_f4(k), cand_f4 = lds_cand_f4(k), cols = k.slots * k.N;
+    const int per_wave_f4 = 4 + 16 + cols + dec_f4 + cand_f4 + k.slots * k.list_cap * entry_f4;
     float4 *wbase = smem + lds_p_f4(k) + dec_f4 + (threadIdx.x >> 6) * per_wave_f4;
     L.Pm = Pm;
     L.dec = dec;
     L.cnt = (lds_counter *)reinterpret_cast<int *>(wbase);
     L.cell = wbase + 4;
-    L.cand = reinterpret_cast<int *>(wbase + 20);
-    L.lst = wbase + 20 + dec_f4;
+    L.col = wbase + 20;
+    L.alive = reinterpret_cast<int *>(wbase + 20 + cols);
+    L.cand = reinterpret_cast<unsigned *>(wbase + 20 + cols + dec_f4);
+    L.lst = wbase + 20 + cols + dec_f4 + cand_f4;
     for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
         Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
-    for (int i = threadIdx.x; i < k.slots * k.NZ; i += blockDim.x) {
-        const int slot = i / k.NZ, s = i - slot * k.NZ;
-        const int cam = s / k.gz, iz = s - cam * k.gz;
-        dec[i] = (slot << 28) | (cam << 16) | iz;
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        const int slot = i / k.N, cam = i - slot * k.N;
+        dec[i] = (slot << 28) | (cam << 16);
     }
     __syncthreads();
     return L;
@@ -367,11 +378,16 @@ enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3 };
 // the exact test it would otherwise take (and fail).
 constexpr float kEarlySlack = 1.0e-3f;
 
-// Phase A of one round of a wavefront: the samples of its `slots` cells, in two stages.
-//   stage 1  all slots*NZ samples, lanes = samples: the three dot products and a division-free
-//            test that can only reject samples the exact test rejects too (behind the camera,
-//            or outside the image by more than kEarlySlack).  About 80 % of all samples end
-//            here.  Survivors are compacted, in order, into the candidate list.
+// Phase A of one round of a wavefront: the samples of its `slots` cells, in three stages.
+//   stage 0  lanes = (cell, camera) columns: the (x, y) part of the three dot products, shared by
+//            the column's height bins, and a test of the column's two end bins.  U, V and D are
+//            monotone in the height bin (every rounded operation is), so a column whose end bins
+//            both miss the image on the same side, or both lie behind the camera, holds no sample
+//            that stage 1 could pass.  About three columns in four end here.
+//   stage 1  lanes = height bins of the remaining columns: the rest of the dot products and a
+//            division-free test that can only reject samples the exact test rejects too (behind
+//            the camera, or outside the image by more than kEarlySlack).  Survivors are compacted,
+//            in order, into the candidate list.
 //   stage 2  lanes = candidates, densely packed: the canonical arithmetic (divisions, floor,
 //            bilinear weights), the depth model, the weight threshold; what is kept goes, still
 //            in (camera, height) order, into its slot's entry list.
@@ -381,7 +397,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                                         int lane, const int *__restrict__ chunk_prefix = nullptr,
                                         int *__restrict__ cursor = nullptr, int pair_cap = 0) {
     constexpr bool BACKWARD = MODE == kModeScatter || MODE == kModeFill;
-    const int total = k.slots * k.NZ;
+    const int n_cols = k.slots * k.N;
     if (lane < 16) L.cnt[lane] = 0;
     if (lane < k.slots) {
         int ix = 0, iy = 0;
@@ -392,29 +408,64 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
-    // ---- stage 1
-    int n_cand = 0;
     const float u_max = k.Wi_f * (1.0f + kEarlySlack), v_max = k.Hi_f * (1.0f + kEarlySlack);
-    for (int base = 0; base < total; base += kWave) {
-        const int idx = base + lane;
-        bool pass = false;
-        if (idx < total) {
-            const int d = L.dec[idx];
-            const float4 c = L.cell[(d >> 28) & 15];
+    // ---- stage 0
+    int n_alive = 0;
+    const float z_first = voxel_coord(k.zmin, 0, k.vz), z_last = voxel_coord(k.zmin, k.gz - 1, k.vz);
+    for (int base = 0; base < n_cols; base += kWave) {
+        const int cc = base + lane;
+        bool alive = false;
+        if (cc < n_cols) {
+            const int code = L.dec[cc];
+            const float4 c = L.cell[(code >> 28) & 15];
             if (c.z != 0.0f) {
-                const float *P = L.Pm + ((d >> 16) & 0xfff) * 12;
-                const float x = c.x, y = c.y, z = voxel_coord(k.zmin, d & 0xffff, k.vz);
-                const float D = ((P[8] * x + P[9] * y) + P[10] * z) + P[11];
-                if (D > 0.0f) {
-                    const float U = ((P[0] * x + P[1] * y) + P[2] * z) + P[3];
-                    const float V = ((P[4] * x + P[5] * y) + P[6] * z) + P[7];
-                    const float dc = fmaxf(D, k.eps), lo = -kEarlySlack * dc;
-                    pass = U >= lo && U <= u_max * dc && V >= lo && V <= v_max * dc;
+                const float *P = L.Pm + ((code >> 16) & 0xfff) * 12;
+                const float au = P[0] * c.x + P[1] * c.y, av = P[4] * c.x + P[5] * c.y, ad = P[8] * c.x + P[9] * c.y;
+                L.col[cc] = make_float4(au, av, ad, __int_as_float(code));
+                const float d0 = (ad + P[10] * z_first) + P[11], d1 = (ad + P[10] * z_last) + P[11];
+                const float d_hi = fmaxf(d0, d1);
+                if (d_hi > 0.0f) {
+                    const float u0 = (au + P[2] * z_first) + P[3], u1 = (au + P[2] * z_last) + P[3];
+                    const float v0 = (av + P[6] * z_first) + P[7], v1 = (av + P[6] * z_last) + P[7];
+                    // stage 1 compares every bin with bounds that grow with its clamped depth
+                    const float dc = fmaxf(d_hi, k.eps), lo = -kEarlySlack * dc;
+                    alive = fmaxf(u0, u1) >= lo && fminf(u0, u1) <= u_max * dc && fmaxf(v0, v1) >= lo &&
+                            fminf(v0, v1) <= v_max * dc;
                 }
             }
         }
+        const unsigned long long m = __ballot(alive);
+        if (alive) L.alive[n_alive + __popcll(m & lanemask_lt(lane))] = cc;
+        n_alive += __popcll(m);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- stage 1
+    int n_cand = 0;
+    const int total = n_alive * k.gz;
+    for (int base = 0; base < total; base += kWave) {
+        const int idx = base + lane;
+        bool pass = false;
+        unsigned key = 0;
+        if (idx < total) {
+            const int a = (int)(__umul24((unsigned)idx, (unsigned)k.gz_magic) >> k.gz_shift);
+            const int iz = idx - a * k.gz;
+            const int cc = L.alive[a];
+            const float4 col = L.col[cc];
+            const float *P = L.Pm + ((__float_as_int(col.w) >> 16) & 0xfff) * 12;
+            const float z = voxel_coord(k.zmin, iz, k.vz);
+            const float D = (col.z + P[10] * z) + P[11];
+            key = ((unsigned)cc << 16) | (unsigned)iz;
+            if (D > 0.0f) {
+                const float U = (col.x + P[2] * z) + P[3];
+                const float V = (col.y + P[6] * z) + P[7];
+                const float dc = fmaxf(D, k.eps), lo = -kEarlySlack * dc;
+                pass = U >= lo && U <= u_max * dc && V >= lo && V <= v_max * dc;
+            }
+        }
         const unsigned long long m = __ballot(pass);
-        if (pass) L.cand[n_cand + __popcll(m & lanemask_lt(lane))] = idx;
+        if (pass) L.cand[n_cand + __popcll(m & lanemask_lt(lane))] = key;
         n_cand += __popcll(m);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -424,7 +475,9 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
     for (int base = 0; base < n_cand; base += kWave) {
         const int j = base + lane;
         const bool active = j < n_cand;
-        const int d = active ? L.dec[L.cand[j]] : 0;
+        const unsigned key = active ? L.cand[j] : 0u;
+        const float4 col = active ? L.col[key >> 16] : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int d = __float_as_int(col.w);
         const int slot = active ? (d >> 28) & 15 : 16 + (lane & 1);   // idle lanes: no real slot
         const int cam = (d >> 16) & 0xfff;
         float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w2 = w0;
@@ -434,7 +487,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         if (active) {
             const float4 c = L.cell[slot];
             cellxy = __float_as_int(c.w);
-            Geom g = project_sample(k, L.Pm + cam * 12, c.x, c.y, voxel_coord(k.zmin, d & 0xffff, k.vz));
+            Geom g = project_column(k, L.Pm + cam * 12, col.x, col.y, col.z, voxel_coord(k.zmin, key & 0xffffu, k.vz));
             if (g.valid) {
                 float w00 = (1.0f - g.du) * (1.0f - g.dv);
                 float w01 = (1.0f - g.du) * g.dv;
@@ -579,8 +632,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
-        int ix = 0, iy = 0;
-        bool mine = carrier && cell_of(k, q0 + slot, ix, iy);
+        // phase A left the slot's cell in LDS: valid flag and ix | iy << 16
+        const float4 mycell = L.cell[carrier ? slot : 0];
+        const int ix = __float_as_int(mycell.w) & 0xffff, iy = __float_as_int(mycell.w) >> 16;
+        const bool mine = carrier && mycell.z != 0.0f;
         const int n = mine ? cnt[slot] : 0;
         const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * 2;
         // the number of samples that enter the mean; the backward pass can reuse it
@@ -643,15 +698,16 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
             }
             for (; e < n; ++e) gather(e);
             if (mine) {
-                const float nf = (float)n;
+                // the mean as a product with 1/n (one division per cell instead of one per channel;
+                // it can differ from the quotient in the last place)
+                const float scale = k.reduce_sum ? 1.0f : (n > 0 ? 1.0f / (float)n : 0.0f);
 #pragma unroll
                 for (int j = 0; j < CPL; ++j) {
                     int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
                     if (ch < k.C) {
                         float res[VEC];
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v)
-                            res[v] = k.reduce_sum ? acc[j][v] : (n > 0 ? acc[j][v] / nf : 0.0f);
+                        for (int v = 0; v < VEC; ++v) res[v] = acc[j][v] * scale;
                         if (VEC == 1) {
                             o[ch] = res[0];
                         } else {
@@ -1952,10 +2008,20 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     k.blocks_per_batch = (k.padded_cells + cells_per_block - 1) / cells_per_block;
     k.n_blocks = k.blocks_per_batch * k.B;
     const size_t p_f4 = (size_t)(k.N * 12 + 3) / 4;
-    const size_t dec_f4 = ((size_t)k.slots * k.NZ + 3) / 4;
+    const size_t cols = (size_t)k.slots * k.N, dec_f4 = (cols + 3) / 4;
+    const size_t cand_f4 = ((size_t)k.slots * k.NZ + 3) / 4;
     auto block_lds = [&](int entry_f4) {
-        return (p_f4 + dec_f4 + (size_t)waves * (20 + dec_f4 + (size_t)k.slots * k.list_cap * entry_f4)) * 16;
+        return (p_f4 + dec_f4 +
+                (size_t)waves * (20 + cols + dec_f4 + cand_f4 + (size_t)k.slots * k.list_cap * entry_f4)) * 16;
     };
+    {
+        // exact division of a sample index below 4096 by gz: multiply and shift
+        if ((long long)k.slots * k.NZ >= 4096) return FBEV_ERR_TOO_LARGE;
+        int l = 0;
+        while ((1 << l) < k.gz) ++l;
+        k.gz_shift = 12 + l;
+        k.gz_magic = (int)((((long long)1 << k.gz_shift) + k.gz - 1) / k.gz);
+    }
     plan->lds_fwd = block_lds(2);
     plan->lds_bwd = block_lds(2);
     plan->lds_fill = block_lds(3);
