@@ -89,7 +89,7 @@ constexpr int kReplicas = 1 << kReplicaBits;
 // With fixed-capacity segments (no counting pass) a texel has one segment per wavefront of the
 // block that later gathers it.
 constexpr int kFixedReplicas = 4;
-constexpr int kFixedMinSegment = 16;          // shorter segments would mostly overflow: count instead
+constexpr int kFixedMinSegment = 4;           // shorter segments would mostly overflow: count instead
 static_assert(kFixedReplicas == 4, "the texel pass reads a texel's claim counters as one int4");
 constexpr int kScanChunkBits = 12;           // counters are prefix-summed in chunks of 4096
 
@@ -369,8 +369,8 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 //   backward  word 0: du, dv, t00, (u1 != u0) | (v1 != v0) << 1 -- the four weights and texels
 //                     follow from these exactly as phase A computed them
 //             word 1: wgt, a, b, (k0 | k1 << 16)
-//             word 2 (inverse map only): for each corner the position of its (cell, coefficient)
-//                     pair in the texel-sorted pair array, or -1 if the array is full
+//             word 2 (inverse map only): .x the position of the sample's pair in the pair array
+//                     (sorted by first corner texel), or -1 if the array is full
 enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3 };
 
 // Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
@@ -512,34 +512,21 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         }
         const int prev_slot = __shfl_up(slot, 1, kWave);
         // Consecutive height bins of one (cell, camera) often fall on the same texel (far cells
-        // compress onto the horizon rows).  Corners that repeat the texel of the previous kept
-        // sample of the same cell form a run; when counting, the run's first lane adds the whole
-        // run with ONE atomic.  (Claiming positions per run as well was measured: the shuffles
-        // cost the cell pass more than the saved returning atomics.)
-        int run_lead[4] = {lane, lane, lane, lane}, run_len[4] = {1, 1, 1, 1};
+        // compress onto the horizon rows).  Samples that repeat the first corner of the previous
+        // kept sample of the same cell form a run; when counting, the run's first lane adds the
+        // whole run with ONE atomic.  (Claiming positions per run as well was measured: the
+        // shuffles cost the cell pass more than the saved returning atomics.)
         if (MODE == kModeCount) {
             const int prev_keep = __shfl_up((int)keep, 1, kWave);
-            const bool chain = keep && lane > 0 && prev_keep != 0 && prev_slot == slot;
-            const int tc[4] = {tx.x, tx.y, tx.z, tx.w};
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const bool cont = __shfl_up(tc[c], 1, kWave) == tc[c] && chain;
-                const unsigned long long cm = __ballot(cont);
-                // first lane of my run: the highest lane at or below me that does not continue
-                run_lead[c] = 63 - __clzll(~cm & lanemask_le(lane));
-                // lanes after me that continue without a gap
-                const unsigned long long after = lane == 63 ? 0ull : (cm >> (lane + 1));
-                run_len[c] = 1 + (~after == 0ull ? 63 - lane : __ffsll((long long)~after) - 1);
-            }
-        }
-        if (MODE == kModeCount) {
-            if (keep) {
-                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
-                if (run_lead[0] == lane) atomicAdd(cursor + tx.x * kReplicas + rep, run_len[0]);
-                if (run_lead[1] == lane) atomicAdd(cursor + tx.y * kReplicas + rep, run_len[1]);
-                if (run_lead[2] == lane) atomicAdd(cursor + tx.z * kReplicas + rep, run_len[2]);
-                if (run_lead[3] == lane) atomicAdd(cursor + tx.w * kReplicas + rep, run_len[3]);
-            }
+            const bool cont = keep && lane > 0 && prev_keep != 0 && prev_slot == slot && __shfl_up(tx.x, 1, kWave) == tx.x;
+            const unsigned long long cm = __ballot(cont);
+            // first lane of my run: the highest lane at or below me that does not continue
+            const int run_lead = 63 - __clzll(~cm & lanemask_le(lane));
+            // lanes after me that continue without a gap
+            const unsigned long long after = lane == 63 ? 0ull : (cm >> (lane + 1));
+            const int run_len = 1 + (~after == 0ull ? 63 - lane : __ffsll((long long)~after) - 1);
+            if (keep && run_lead == lane)
+                atomicAdd(cursor + tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16), run_len);
             continue;
         }
         // candidates are in sample order, so the lanes of one slot are contiguous: [lo, hi)
@@ -559,43 +546,21 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                                           __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
         }
         if (MODE == kModeFill && keep) {
-            // claim one position per corner in the texel's segment of the pair array; the four
-            // requests of all lanes are in flight together, so the round trip is paid once
-            int p0, p1, p2, p3;
+            // claim the sample's position in the list of its first corner texel
+            int pos;
             if (chunk_prefix != nullptr) {
                 // counted segments: cursor holds each segment's start within its scan chunk
-                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
-                const int i0 = tx.x * kReplicas + rep, i1 = tx.y * kReplicas + rep;
-                const int i2 = tx.z * kReplicas + rep, i3 = tx.w * kReplicas + rep;
-                p0 = atomicAdd(cursor + i0, 1);
-                p1 = atomicAdd(cursor + i1, 1);
-                p2 = atomicAdd(cursor + i2, 1);
-                p3 = atomicAdd(cursor + i3, 1);
-                p0 += chunk_prefix[i0 >> kScanChunkBits];
-                p1 += chunk_prefix[i1 >> kScanChunkBits];
-                p2 += chunk_prefix[i2 >> kScanChunkBits];
-                p3 += chunk_prefix[i3 >> kScanChunkBits];
-                p0 = p0 < pair_cap ? p0 : -1;
-                p1 = p1 < pair_cap ? p1 : -1;
-                p2 = p2 < pair_cap ? p2 : -1;
-                p3 = p3 < pair_cap ? p3 : -1;
+                const int i0 = tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16);
+                pos = atomicAdd(cursor + i0, 1) + chunk_prefix[i0 >> kScanChunkBits];
+                pos = pos < pair_cap ? pos : -1;
             } else {
                 // fixed segments of pair_cap pairs per (texel, replica): cursor counts from zero
-                const int rep = replica_of(cellxy & 0xffff, cellxy >> 16) & (kFixedReplicas - 1);
-                const int i0 = tx.x * kFixedReplicas + rep, i1 = tx.y * kFixedReplicas + rep;
-                const int i2 = tx.z * kFixedReplicas + rep, i3 = tx.w * kFixedReplicas + rep;
-                p0 = atomicAdd(cursor + i0, 1);
-                p1 = atomicAdd(cursor + i1, 1);
-                p2 = atomicAdd(cursor + i2, 1);
-                p3 = atomicAdd(cursor + i3, 1);
-                p0 = p0 < pair_cap ? i0 * pair_cap + p0 : -1;
-                p1 = p1 < pair_cap ? i1 * pair_cap + p1 : -1;
-                p2 = p2 < pair_cap ? i2 * pair_cap + p2 : -1;
-                p3 = p3 < pair_cap ? i3 * pair_cap + p3 : -1;
+                const int i0 = tx.x * kFixedReplicas + (replica_of(cellxy & 0xffff, cellxy >> 16) & (kFixedReplicas - 1));
+                pos = atomicAdd(cursor + i0, 1);
+                pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
             }
             float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
-            e[ENTRY_F4 - 1] = make_float4(__int_as_float(p0), __int_as_float(p1), __int_as_float(p2),
-                                          __int_as_float(p3));
+            e[ENTRY_F4 - 1] = make_float4(__int_as_float(pos), 0.f, 0.f, 0.f);
         }
         if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
     }
@@ -735,11 +700,18 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
 //                pass, no floating-point atomics, each gradient row written once.
 __device__ __forceinline__ void atomic_add_f32(float *p, float v) { unsafeAtomicAdd(p, v); }
 
-struct Pair {      // 16 bytes
-    int cell;      // row of grad_out: (b * gy + iy) * gx + ix
-    float coef;    // d out[cell, c] / d feats[texel, c]
-    float da, db;  // this sample's contribution to d_depth[texel, 0] and [texel, 1] (parametric models)
+// One record per kept sample, filed under the sample's first corner texel (v0, u0): the texel
+// pass of a texel reads the lists of the (up to) four texels whose samples can reach it.
+struct Pair {       // 32 bytes
+    int cell;       // row of grad_out: (b * gy + iy) * gx + ix, shifted left by bin_bits with the depth bin below
+    float coef;     // depth weight (/ count for the mean): d out[cell, c] / d feats[corner, c] is coef * corner weight
+    float du, dv;   // bilinear fractions
+    float ga, gb;   // <grad_out, sampled feature> * (d weight / d depth parameter); times the corner weight it is
+                    // the sample's contribution to d_depth[corner, 0 / 1] (parametric) or [corner, k0 / k1]
+    int flags;      // bit 0: u1 != u0, bit 1: v1 != v0 (clamped at the last column / row otherwise)
+    int pad;
 };
+static_assert(sizeof(Pair) == 32, "a pair is written as two 16-byte words");
 
 // Zero up to three regions of 32-bit words in one launch (segment counters and, when the
 // library is asked to, the two gradient buffers).  A kernel rather than hipMemsetAsync, so the
@@ -970,12 +942,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 const unsigned r00 = (unsigned)t00 * (unsigned)k.row_units;
                 const unsigned r01 = r00 + ((fl & 2) ? row_step_v : 0u);
                 const unsigned r10 = r00 + ((fl & 1) ? (unsigned)k.row_units : 0u), r11 = r01 + (r10 - r00);
-                bool s00 = true, s01 = true, s10 = true, s11 = true;
-                if (FILL) {
-                    const float4 pf = my[EF4 * e + 2];
-                    s00 = __float_as_int(pf.x) < 0; s01 = __float_as_int(pf.y) < 0;
-                    s10 = __float_as_int(pf.z) < 0; s11 = __float_as_int(pf.w) < 0;
-                }
+                // scatter path, or a sample without room in the pair array: atomics for all four corners
+                const bool spill = FILL ? __float_as_int(my[EF4 * e + 2].x) < 0 : true;
+                const bool s00 = spill, s01 = spill, s10 = spill, s11 = spill;
                 const float a00 = w00 * wgt, a01 = w01 * wgt, a10 = w10 * wgt, a11 = w11 * wgt;
 #pragma unroll
                 for (int j = 0; j < CPL; ++j) {
@@ -1072,37 +1041,36 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 }
             }
             if (FILL && first_pass) {
-                // ---- the pairs of this round: lanes = (entry, corner), every slot in turn
+                // ---- the pairs of this round: the lanes of a slot take the slot's entries in turn
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
-                for (int sl = 0; sl < k.slots; ++sl) {
-                    const int ns = cnt[sl];
-                    if (ns == 0) continue;
-                    const int cxy = __float_as_int(L.cell[sl].w);
-                    const int pcell = (b * k.gy + (cxy >> 16)) * k.gx + (cxy & 0xffff);
-                    const float pinv = k.reduce_sum ? 1.0f : 1.0f / (float)ns;
-                    const float4 *lst_s = lst + (size_t)sl * k.list_cap * EF4;
-                    for (int i = lane; i < ns * 4; i += kWave) {
-                        const int pe = i >> 2, c = i & 3;
-                        const float4 geo = lst_s[EF4 * pe], dwp = lst_s[EF4 * pe + 1], pfp = lst_s[EF4 * pe + 2];
-                        const float du = geo.x, dv = geo.y;
-                        // corner c: 0 (v0,u0) 1 (v1,u0) 2 (v0,u1) 3 (v1,u1); same products as phase A
-                        const float wu = (c & 2) ? du : 1.0f - du, wv = (c & 1) ? dv : 1.0f - dv;
-                        const float wcc = wu * wv;
-                        const int posc = __float_as_int(c == 0 ? pfp.x : (c == 1 ? pfp.y : (c == 2 ? pfp.z : pfp.w)));
-                        // G * a and G * b (G already carries 1/count)
-                        const float da = fold ? dwp.y * wcc : 0.0f, db = fold ? dwp.z * wcc : 0.0f;
+                {
+                    const int pcell = cell;
+                    const float pinv = inv;
+                    const float4 *lst_s = my;
+                    for (int pe = lis; pe < n; pe += k.lanes_per_slot) {
+                        const float4 geo = lst_s[EF4 * pe], dwp = lst_s[EF4 * pe + 1];
+                        const int posp = __float_as_int(lst_s[EF4 * pe + 2].x);
                         const int kk = __float_as_int(dwp.w);
                         const int k0 = parametric ? 0 : (kk & 0xffff), k1 = parametric ? 1 : (kk >> 16);
-                        if (posc >= 0) {
+                        // G * a and G * b (G already carries 1/count)
+                        const float ga = fold ? dwp.y : 0.0f, gb = fold ? dwp.z : 0.0f;
+                        if (posp >= 0) {
                             const int word = fold ? ((pcell << k.bin_bits) | k0) : pcell;
-                            *reinterpret_cast<float4 *>(pairs + posc) =
-                                make_float4(__int_as_float(word), wcc * dwp.x * pinv, da, db);
+                            float4 *dst = reinterpret_cast<float4 *>(pairs + posp);
+                            dst[0] = make_float4(__int_as_float(word), dwp.x * pinv, geo.x, geo.y);
+                            dst[1] = make_float4(ga, gb, geo.w, 0.0f);
                         } else if (fold) {
+                            const float du = geo.x, dv = geo.y;
                             const int fl = __float_as_int(geo.w);
-                            const int tt = __float_as_int(geo.z) + ((c & 1) && (fl & 2) ? k.W : 0) + ((c & 2) ? (fl & 1) : 0);
-                            atomic_add_f32(d_depth + (size_t)tt * Dd + k0, da);
-                            atomic_add_f32(d_depth + (size_t)tt * Dd + k1, db);
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) {
+                                // corner c: 0 (v0,u0) 1 (v1,u0) 2 (v0,u1) 3 (v1,u1); same products as phase A
+                                const float wcc = ((c & 2) ? du : 1.0f - du) * ((c & 1) ? dv : 1.0f - dv);
+                                const int tt = __float_as_int(geo.z) + ((c & 1) && (fl & 2) ? k.W : 0) + ((c & 2) ? (fl & 1) : 0);
+                                atomic_add_f32(d_depth + (size_t)tt * Dd + k0, ga * wcc);
+                                atomic_add_f32(d_depth + (size_t)tt * Dd + k1, gb * wcc);
+                            }
                         }
                     }
                 }
@@ -1112,12 +1080,14 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     }
 }
 
-// Texel pass of the inverse-map backward.  A texel's pairs are handled by one block, or, when
-// the grid has a second dimension and there are more than kTexelPart of them, by up to
-// gridDim.y blocks that each take an equal share.  Every block of a texel first has to read the
-// texel's segment bounds, so idle blocks are not free: the host splits only when there are too
-// few texels to fill the machine otherwise (kTexelSplitBelow).  A block's
-// 4 * (64 / lanes_per_row) workers stride over its pairs, each gathering grad_out rows with
+// Texel pass of the inverse-map backward.  The samples that reach texel t are filed under their
+// first corner: t itself, its left neighbour, the texel above, and the one above-left (a sample's
+// corners are (v0|v1, u0|u1) with u1 = u0 + 1 and v1 = v0 + 1 unless clamped).  Those four lists
+// are handled by one block, or, when the grid has a second dimension and a list is longer than
+// kTexelPart, by up to gridDim.y blocks that each take an equal share of every list.  Every block
+// of a texel first has to read the lists' bounds, so idle blocks are not free: the host splits
+// only when there are too few texels to fill the machine otherwise (kTexelSplitBelow).  A block's
+// WAVES * (64 / lanes_per_row) workers stride over the pairs, each gathering grad_out rows with
 // 128-bit loads; partial rows meet in LDS.  A texel handled by one block is updated with plain
 // loads and stores; the shares of a split texel are combined with fp32 atomics (at most
 // gridDim.y per address).
@@ -1125,54 +1095,67 @@ constexpr int kTexelMaxSplit = 8;
 constexpr int kTexelSplitBelow = 8192;
 constexpr int kTexelPart = 128;
 constexpr int kTexelNarrowFrom = 50000;
-constexpr int kTexelNarrowPairs = 2048;      // upper bound of pairs per texel: four per sample
+constexpr int kTexelNarrowPairs = 512;       // upper bound of samples per list
+constexpr int kTexelSegs = 4 * kFixedReplicas;   // lists of a texel with fixed segments: 4 first corners x replicas
 template <int VEC, int WAVES>
 __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
     const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
     float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs) {
     extern __shared__ float4 smem[];
-    float *part = reinterpret_cast<float *>(smem);
+    // [kTexelSegs list starts][kTexelSegs list ends][kTexelSegs + 1 (+ 3) positions in the sequence][partial rows ...]
+    int *seg_lo = reinterpret_cast<int *>(smem);
+    int *seg_hi = seg_lo + kTexelSegs;
+    int *seg_pre = seg_hi + kTexelSegs;
+    float *part = reinterpret_cast<float *>(seg_pre + kTexelSegs + 4);
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
-    constexpr int n_waves = WAVES, kSegs = kFixedReplicas / WAVES;
-    // this wavefront's pairs: n_segs segments [seg_start[i], seg_end_[i]) walked in steps of wave_stride
-    int seg_start[kSegs], seg_end_[kSegs], n_segs = 0, wave_stride;
-    bool shared_texel;
-    if (chunk_prefix != nullptr) {
-        // counted segments, one after the other: from the end of the previous texel's last
-        // replica to the end of this texel's; the wavefronts interleave
-        const long long first = (long long)t * kReplicas - 1, last = (long long)t * kReplicas + kReplicas - 1;
-        int start = t == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
-        int end = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
-        if (start >= end) return;      // uniform for the block
-        const int n_all = end - start;
-        const int n_parts = min((int)gridDim.y, (n_all + kTexelPart - 1) / kTexelPart);
-        if ((int)blockIdx.y >= n_parts) return;
-        seg_start[0] = start + (int)(((long long)n_all * blockIdx.y) / n_parts) + wave * kWave;
-        seg_end_[0] = start + (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
-        n_segs = 1;
-        wave_stride = n_waves * kWave;
-        shared_texel = n_parts > 1;
-    } else {
-        // fixed segments of pair_cap pairs, dealt to the wavefronts in turn; seg_end holds how many were claimed
-        const int4 c = *reinterpret_cast<const int4 *>(seg_end + (size_t)t * kFixedReplicas);
-        const int n_max = min(max(max(c.x, c.y), max(c.z, c.w)), pair_cap);
-        const int n_parts = min((int)gridDim.y, (n_max + kTexelPart - 1) / kTexelPart);
-        if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
-#pragma unroll
-        for (int i = 0; i < kSegs; ++i) {
-            const int r = wave + i * WAVES;          // wavefront w takes segments w, w + WAVES, ...
-            const int mine = min(r == 0 ? c.x : (r == 1 ? c.y : (r == 2 ? c.z : c.w)), pair_cap);
-            const int base = (t * kFixedReplicas + r) * pair_cap;
-            seg_start[i] = base + (int)(((long long)mine * blockIdx.y) / n_parts);
-            seg_end_[i] = base + (int)(((long long)mine * (blockIdx.y + 1)) / n_parts);
+    constexpr int n_waves = WAVES;
+    const bool counted = chunk_prefix != nullptr;
+    // List e of the texel: first corner (e & 3 with fixed segments, e when counted): bit 0 = one
+    // texel to the left, bit 1 = one row up; replica e >> 2 with fixed segments.  A cell's samples
+    // on neighbouring height bins sit in different lists of the same replica, at about the same
+    // relative position (they were claimed together): replica-major order keeps them close in
+    // time, so the second gather of the cell's grad_out row finds it in cache.
+    const int tu = t % k.W, tv = (t / k.W) % k.H;
+    if (threadIdx.x < kTexelSegs) {
+        const int e = threadIdx.x;
+        const int o = counted ? e : e & 3;
+        const bool exists = (counted ? e < 4 : true) && (!(o & 1) || tu > 0) && (!(o & 2) || tv > 0);
+        const int q = t - (o & 1) - ((o & 2) ? k.W : 0);
+        int lo = 0, hi = 0;
+        if (exists && counted) {
+            // counted segments, one after the other: from the end of the previous texel's last
+            // replica to the end of this texel's
+            const long long first = (long long)q * kReplicas - 1, last = (long long)q * kReplicas + kReplicas - 1;
+            lo = q == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
+            hi = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
+        } else if (exists) {
+            // fixed segments of pair_cap pairs; seg_end holds how many were claimed
+            const int i = q * kFixedReplicas + (e >> 2);
+            lo = i * pair_cap;
+            hi = lo + min(seg_end[i], pair_cap);
         }
-        n_segs = kSegs;
-        wave_stride = kWave;
-        shared_texel = n_parts > 1;
+        seg_lo[e] = lo;
+        seg_hi[e] = max(hi, lo);
     }
+    __syncthreads();
+    // the lists one after the other form one sequence of pairs; seg_pre[e] is where list e starts in it
+    if (threadIdx.x <= kTexelSegs) {
+        int before = 0;
+        for (int e = 0; e < (int)threadIdx.x; ++e) before += seg_hi[e] - seg_lo[e];
+        seg_pre[threadIdx.x] = before;
+    }
+    __syncthreads();
+    const int n_all = seg_pre[kTexelSegs];
+    const int n_parts = min((int)gridDim.y, (n_all + 4 * kTexelPart - 1) / (4 * kTexelPart));
+    if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
+    const bool shared_texel = n_parts > 1;
+    const int part_lo = (int)(((long long)n_all * blockIdx.y) / n_parts);
+    const int part_hi = (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
+    // the wavefronts take chunks of the sequence in turn: 64 pairs, fewer when that leaves a wavefront idle
+    const int chunk = min(kWave, max(1, (part_hi - part_lo + n_waves - 1) / n_waves));
     const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
     const int wpw = kWave / lanes_per_row;            // workers per wavefront
     const int nw = wpw * n_waves;
@@ -1205,28 +1188,47 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
         // load, and hands them to its workers through lane shuffles; four grad_out rows per
         // worker are in flight before the first is used.  The loop is bound by load latency:
         // without this the pair load and the row load it addresses form a dependent chain.
+        for (int bstart = part_lo + wave * chunk; bstart < part_hi; bstart += n_waves * chunk) {
+            const int nb = min(chunk, part_hi - bstart);
+            float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f), pd = make_float4(0.f, 0.f, 0.f, 0.f);
+            int o = 0;
+            if (lane < nb) {
+                // which list position bstart + lane falls into, and where that is in the pair array
+                const int vi = bstart + lane;
+                int e = 0;
 #pragma unroll
-        for (int sg = 0; sg < kSegs; ++sg)
-        for (int bstart = sg < n_segs ? seg_start[sg] : 0; sg < n_segs && bstart < seg_end_[sg]; bstart += wave_stride) {
-            const int nb = min(kWave, seg_end_[sg] - bstart);
-            float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f);
-            if (lane < nb) pr = *reinterpret_cast<const float4 *>(pairs + bstart + lane);
+                for (int j = 1; j < kTexelSegs; ++j) e += vi >= seg_pre[j] ? 1 : 0;
+                o = counted ? e : e & 3;
+                const float4 *src = reinterpret_cast<const float4 *>(pairs + seg_lo[e] + (vi - seg_pre[e]));
+                pr = src[0];
+                pd = src[1];
+            }
             const int word = __float_as_int(pr.x);
             // a pair is written by the cell pass before this kernel starts; the range check only
             // keeps a logic error from turning into a wild read (such a pair counts as cell 0
             // with coefficient 0)
             const bool valid = (unsigned)(word >> bin_bits) < n_cells;
+            // the sample's bilinear weight on this texel: the corners that land here (a clamped
+            // corner stays on the first corner's column / row)
+            const float du = pr.z, dv = pr.w;
+            const bool fu = __float_as_int(pd.z) & 1, fv = __float_as_int(pd.z) & 2;
+            const float w00 = (1.0f - du) * (1.0f - dv), w01 = (1.0f - du) * dv, w10 = du * (1.0f - dv), w11 = du * dv;
+            float cw;
+            if (o == 0) cw = w00 + (fu ? 0.0f : w10) + (fv ? 0.0f : w01) + ((fu || fv) ? 0.0f : w11);
+            else if (o == 1) cw = fu ? w10 + (fv ? 0.0f : w11) : 0.0f;
+            else if (o == 2) cw = fv ? w01 + (fu ? 0.0f : w11) : 0.0f;
+            else cw = (fu && fv) ? w11 : 0.0f;
             // where the pair's grad_out row starts, in units of 16 bytes (one float off the vector path)
             const unsigned my_row = valid ? (unsigned)(word >> bin_bits) * out_units : 0u;
-            const float my_coef = valid ? pr.y : 0.0f;
+            const float my_coef = valid ? pr.y * cw : 0.0f;
             if (c0 == 0 && valid) {
                 if (bin_sums) {
                     const int k0 = word & bin_mask;
-                    __hip_atomic_fetch_add(bins + k0, pr.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(bins + min(k0 + 1, k.Dd - 1), pr.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(bins + k0, pd.x * cw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(bins + min(k0 + 1, k.Dd - 1), pd.y * cw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 } else {
-                    sa += pr.z;
-                    sb += pr.w;
+                    sa += pd.x * cw;
+                    sb += pd.y * cw;
                 }
             }
             // Full groups of UNR pairs per worker run without predicates (lanes that carry no
@@ -2264,7 +2266,7 @@ int fbev_backward_columns(const fbev_problem *p, const float *grad_out, const vo
 
 uint64_t fbev_backward_max_pairs(const fbev_problem *p) {
     if (validate(p, true) != FBEV_OK) return 0;
-    return 4ull * (uint64_t)sample_count(p);
+    return (uint64_t)sample_count(p);        // one pair per sample
 }
 
 size_t fbev_backward_workspace_bytes(const fbev_problem *p, uint64_t pair_capacity) {
@@ -2285,7 +2287,7 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const size_t index_bytes = ws_index_bytes(p);
     if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
     // pair positions are 32-bit: every sample corner must be countable
-    if (4 * sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    if (sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
     // the texel pass addresses grad_out rows in 32-bit units (16 bytes, or one float off the vector path)
     const bool rows_vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
     if ((long long)p->batch * p->grid_y * p->grid_x * (rows_vec4 ? p->channels / 4 : p->channels) >= (1ll << 32))
@@ -2342,8 +2344,8 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const int cq = (p->channels + vec - 1) / vec;
     const int lpr = cq < kWave ? cq : kWave;
     // Four wavefronts per texel, or one (taking the four segments in turn) when there are many
-    // texels whose lists cannot be long: measured at 67 584 texels with about 57 pairs each, one
-    // wavefront is 24 % faster than four; at 33 792 texels with about 280 pairs, two are 18 % slower.
+    // texels whose lists cannot be long: measured at 67 584 texels reached by about 57 sample corners
+    // each, one wavefront is 24 % faster than four; at 33 792 texels with about 280, two are 18 % slower.
     const bool short_lists = texels >= kTexelNarrowFrom && fbev_backward_max_pairs(p) / (uint64_t)texels < kTexelNarrowPairs;
     const int texel_waves = short_lists ? 1 : kWavesPerBlock;
     const int nw = (kWave / lpr) * texel_waves;
@@ -2351,8 +2353,8 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     // and room for the depth bin in a pair's first word)
     const int from_pairs =
         (d_depth != nullptr && pl.k.C <= pl.k.lanes_per_slot * pl.vec * pl.cpl && pl.k.bin_bits >= 0) ? 1 : 0;
-    const size_t lds = ((size_t)nw * (lpr * vec + 2) + (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) *
-                       sizeof(float);
+    const size_t lds = ((size_t)nw * (lpr * vec + 2) + (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0) +
+                        3 * kTexelSegs + 4) * sizeof(float);
     long long want_split = kTexelSplitBelow / texels;
     const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);

@@ -48,15 +48,15 @@ def _backward_mode() -> int:
 
 
 def _pair_capacity(batch: int, cams: int, grid) -> int:
-    """Pair slots of the inverse-map workspace.  Room for every sample corner (16 bytes each)
-    lets the library skip its counting passes; FLASHBEV_WORKSPACE_MB (default 16384) bounds the
+    """Pair slots of the inverse-map workspace.  Room for every sample (32 bytes each) lets the
+    library skip its counting passes; FLASHBEV_WORKSPACE_MB (default 16384) bounds the
     allocation, and a smaller workspace is packed exactly instead (-1 = the extension's default,
     room for everything)."""
     limit_mb = float(os.environ.get("FLASHBEV_WORKSPACE_MB", "16384"))
-    max_pairs = 4 * batch * cams * grid[0] * grid[1] * grid[2]
-    if max_pairs * 16 <= limit_mb * 2 ** 20:
+    max_pairs = batch * cams * grid[0] * grid[1] * grid[2]
+    if max_pairs * 32 <= limit_mb * 2 ** 20:
         return -1
-    return max(0, int(limit_mb * 2 ** 20) // 16)
+    return max(0, int(limit_mb * 2 ** 20) // 32)
 
 
 _host_cache: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 3
+#define FBEV_ABI_VERSION 4
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -102,14 +102,16 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
 /*
  * Backward through an inverse map (texel -> contributing samples): the same gradients as
  * fbev_backward, formed without floating-point atomics on the feature gradient.  The cell
- * pass writes one 16-byte (cell, coefficient) pair per sample corner into the texel's segment
- * of the workspace, the texel pass gathers per texel.  `accumulate` as in fbev_backward.
+ * pass writes one 32-byte record ("pair": cell, coefficient, bilinear fractions, depth-gradient
+ * terms) per kept sample into the workspace segment of the sample's first corner texel; the
+ * texel pass of a texel gathers from the segments of the four texels whose samples reach it.
+ * `accumulate` as in fbev_backward.
  * `workspace` is caller-owned device memory, 16-byte aligned, of at least
  * fbev_backward_workspace_bytes(p, 0) bytes, and carries no state between calls.  Its pair
  * capacity selects the layout:
  *   - room for fbev_backward_max_pairs(p) pairs or more: every texel owns fixed segments
  *     (capacity / texels pair slots, in four replicas) and the call is three launches;
- *   - anything smaller: the call first counts the sample corners per texel and prefix-sums
+ *   - anything smaller: the call first counts the samples per first-corner texel and prefix-sums
  *     the counts, so that the pairs are packed exactly (two more passes over the samples).
  * Pairs that find no room (a full segment, or a packed array shorter than the number of
  * pairs) are applied with atomics instead, so any capacity gives correct results.
@@ -143,7 +145,7 @@ int fbev_backward_columns(const fbev_problem *p, const float *grad_out, const vo
 
 size_t fbev_backward_columns_workspace_bytes(const fbev_problem *p);
 
-/* Upper bound of the pairs one backward call can produce: 4 corners per (cell, camera, height) sample. */
+/* Upper bound of the pairs one backward call can produce: one per (cell, camera, height) sample. */
 uint64_t fbev_backward_max_pairs(const fbev_problem *p);
 
 /* Bytes of a workspace holding the per-texel index plus `pair_capacity` pairs. */

@@ -220,7 +220,7 @@ def test_full_size_against_oracle_on_one_batch_element():
 def test_fixed_segments_overflow_falls_back_to_atomics(dist):
     """A distant, narrow grid projects onto a handful of texels: their fixed segments (capacity =
     the average over all texels) overflow by far, and the overflow is applied with atomics."""
-    w = small("cfg1_tiny", channels=16, roi_range=(38.0, 42.0, -1.0, 1.0, 0.5, 2.5), grid_size=(32, 32, 4),
+    w = small("cfg1_tiny", channels=16, roi_range=(38.0, 42.0, -1.0, 1.0, 0.5, 2.5), grid_size=(64, 64, 4),
               depth_bins=64)
     x = make_inputs(w, MODEL[dist], device="cuda", with_grad_out=True)
     p = U.problem_for(x, w, dist, thr=0.0)

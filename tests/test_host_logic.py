@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in flashbev_hip.h but not exported"
     assert sorted(capi.EXPORTS) == names
-    assert lib.fbev_abi_version() == 3
+    assert lib.fbev_abi_version() == 4
     assert lib.fbev_problem_size() == ctypes.sizeof(capi.FbevProblem)
 
 
@@ -91,10 +91,10 @@ def test_validation_status_codes_without_gpu():
 
 def test_workspace_and_byte_helpers():
     p = good_problem()
-    assert capi.backward_max_pairs(p) == 4 * 1 * 5 * 5 * 2 * 2
+    assert capi.backward_max_pairs(p) == 1 * 5 * 5 * 2 * 2
     w0 = capi.backward_workspace_bytes(p, 0)
     assert w0 > 0 and w0 % 256 == 0
-    assert capi.backward_workspace_bytes(p, 100) == w0 + 1600
+    assert capi.backward_workspace_bytes(p, 100) == w0 + 3200
     # compulsory bytes: every operand once
     texels = 1 * 2 * 4 * 6
     fwd = texels * 8 * 4 + texels * 2 * 4 + 2 * 48 + 5 * 5 * 8 * 4
@@ -275,10 +275,10 @@ def test_latency_sweep_harness_selects_experiments_and_keeps_the_reference_schem
 
 
 def test_workspace_limit_selects_the_packed_layout(monkeypatch):
-    """Room for every sample corner by default; a bound in MB turns into a pair capacity."""
+    """Room for every sample by default; a bound in MB turns into a pair capacity."""
     assert op_module._pair_capacity(1, 6, [128, 128, 8]) == -1
     monkeypatch.setenv("FLASHBEV_WORKSPACE_MB", "16")
-    assert op_module._pair_capacity(1, 6, [128, 128, 8]) == 16 * 2 ** 20 // 16       # 50 MB would be needed
+    assert op_module._pair_capacity(1, 6, [128, 128, 8]) == 16 * 2 ** 20 // 32       # 25 MB would be needed
     assert op_module._pair_capacity(1, 1, [32, 32, 4]) == -1
 
 
