@@ -1103,11 +1103,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
     float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs) {
     extern __shared__ float4 smem[];
-    // [kTexelSegs list starts][kTexelSegs list ends][kTexelSegs + 1 (+ 3) positions in the sequence][partial rows ...]
-    int *seg_lo = reinterpret_cast<int *>(smem);
-    int *seg_hi = seg_lo + kTexelSegs;
-    int *seg_pre = seg_hi + kTexelSegs;
-    float *part = reinterpret_cast<float *>(seg_pre + kTexelSegs + 4);
+    float *part = reinterpret_cast<float *>(smem);
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -1118,37 +1114,40 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     // on neighbouring height bins sit in different lists of the same replica, at about the same
     // relative position (they were claimed together): replica-major order keeps them close in
     // time, so the second gather of the cell's grad_out row finds it in cache.
+    // Every wavefront builds the table for itself in its first kTexelSegs lanes (lane e holds list
+    // e): no LDS, no barrier before the first pair is requested.
     const int tu = t % k.W, tv = (t / k.W) % k.H;
-    if (threadIdx.x < kTexelSegs) {
-        const int e = threadIdx.x;
+    int my_lo = 0, my_len = 0;
+    if (lane < kTexelSegs) {
+        const int e = lane;
         const int o = counted ? e : e & 3;
         const bool exists = (counted ? e < 4 : true) && (!(o & 1) || tu > 0) && (!(o & 2) || tv > 0);
         const int q = t - (o & 1) - ((o & 2) ? k.W : 0);
-        int lo = 0, hi = 0;
         if (exists && counted) {
             // counted segments, one after the other: from the end of the previous texel's last
             // replica to the end of this texel's
             const long long first = (long long)q * kReplicas - 1, last = (long long)q * kReplicas + kReplicas - 1;
-            lo = q == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
-            hi = min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap);
+            my_lo = q == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
+            my_len = max(min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap) - my_lo, 0);
         } else if (exists) {
             // fixed segments of pair_cap pairs; seg_end holds how many were claimed
             const int i = q * kFixedReplicas + (e >> 2);
-            lo = i * pair_cap;
-            hi = lo + min(seg_end[i], pair_cap);
+            my_lo = i * pair_cap;
+            my_len = max(min(seg_end[i], pair_cap), 0);
         }
-        seg_lo[e] = lo;
-        seg_hi[e] = max(hi, lo);
     }
-    __syncthreads();
-    // the lists one after the other form one sequence of pairs; seg_pre[e] is where list e starts in it
-    if (threadIdx.x <= kTexelSegs) {
-        int before = 0;
-        for (int e = 0; e < (int)threadIdx.x; ++e) before += seg_hi[e] - seg_lo[e];
-        seg_pre[threadIdx.x] = before;
+    // the lists one after the other form one sequence of pairs; list e starts at my_pre of lane e
+    int my_pre = my_len;
+#pragma unroll
+    for (int off = 1; off < kTexelSegs; off <<= 1) {
+        const int other = __shfl_up(my_pre, off, kWave);
+        if (lane >= off) my_pre += other;
     }
-    __syncthreads();
-    const int n_all = seg_pre[kTexelSegs];
+    my_pre -= my_len;                              // exclusive
+    int list_start[kTexelSegs];                    // wave-uniform copies of the starts of lists 1 ..
+#pragma unroll
+    for (int j = 1; j < kTexelSegs; ++j) list_start[j] = __builtin_amdgcn_readlane(my_pre, j);
+    const int n_all = __builtin_amdgcn_readlane(my_pre, kTexelSegs - 1) + __builtin_amdgcn_readlane(my_len, kTexelSegs - 1);
     const int n_parts = min((int)gridDim.y, (n_all + 4 * kTexelPart - 1) / (4 * kTexelPart));
     if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
     const bool shared_texel = n_parts > 1;
@@ -1191,15 +1190,17 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
         for (int bstart = part_lo + wave * chunk; bstart < part_hi; bstart += n_waves * chunk) {
             const int nb = min(chunk, part_hi - bstart);
             float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f), pd = make_float4(0.f, 0.f, 0.f, 0.f);
-            int o = 0;
-            if (lane < nb) {
-                // which list position bstart + lane falls into, and where that is in the pair array
-                const int vi = bstart + lane;
-                int e = 0;
+            // which list position bstart + lane falls into (all lanes take part in the shuffles;
+            // positions past the chunk fall into some list and are not loaded)
+            const int vi = bstart + lane;
+            int e = 0;
 #pragma unroll
-                for (int j = 1; j < kTexelSegs; ++j) e += vi >= seg_pre[j] ? 1 : 0;
-                o = counted ? e : e & 3;
-                const float4 *src = reinterpret_cast<const float4 *>(pairs + seg_lo[e] + (vi - seg_pre[e]));
+            for (int j = 1; j < kTexelSegs; ++j) e += vi >= list_start[j] ? 1 : 0;
+            const int o = counted ? e : e & 3;
+            // lane e of the wavefront knows where list e lies in the pair array
+            const int src_pos = __shfl(my_lo, e, kWave) + (vi - __shfl(my_pre, e, kWave));
+            if (lane < nb) {
+                const float4 *src = reinterpret_cast<const float4 *>(pairs + src_pos);
                 pr = src[0];
                 pd = src[1];
             }
@@ -2353,8 +2354,8 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     // and room for the depth bin in a pair's first word)
     const int from_pairs =
         (d_depth != nullptr && pl.k.C <= pl.k.lanes_per_slot * pl.vec * pl.cpl && pl.k.bin_bits >= 0) ? 1 : 0;
-    const size_t lds = ((size_t)nw * (lpr * vec + 2) + (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0) +
-                        3 * kTexelSegs + 4) * sizeof(float);
+    const size_t lds = ((size_t)nw * (lpr * vec + 2) + (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) *
+                       sizeof(float);
     long long want_split = kTexelSplitBelow / texels;
     const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);
