@@ -1104,7 +1104,17 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs) {
     extern __shared__ float4 smem[];
     float *part = reinterpret_cast<float *>(smem);
-    const int t = blockIdx.x;
+    // Blocks are dealt to the accelerator dies in turn; let each die walk a contiguous range of
+    // texels, column by column: the texels of a feature-map column gather the cells along one
+    // wedge of rays (a cell's height bins land on neighbouring rows), so their grad_out rows meet
+    // in one L2 while they are still there.
+    // (Measured: 10 % at 33 792 texels with 1 KiB rows; nothing below about 16 000 texels.)
+    int t = blockIdx.x;
+    if (gridDim.x >= 16384) {
+        const int j = xcd_swizzle(blockIdx.x, gridDim.x), hw = k.H * k.W;
+        const int img = j / hw, rem = j - img * hw, u = rem / k.H, v = rem - u * k.H;
+        t = (img * k.H + v) * k.W + u;
+    }
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     constexpr int n_waves = WAVES;
