@@ -368,10 +368,10 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 //                     ((b*N+n)*H + v)*W + u times KParams::row_units) as int bits (t00, t01, t10, t11):
 //                     the gather loop then forms an address with one shift-add, not a 64-bit multiply
 //   backward  word 0: du, dv, t00, (u1 != u0) | (v1 != v0) << 1 -- the four weights and texels
-//                     follow from these exactly as phase A computed them
+//                     follow from these exactly as phase A computed them.  Inverse map: t00 << 2 with
+//                     the two flags below it, and in the fourth place the position of the sample's
+//                     pair in the pair array (sorted by first corner texel), or -1 if the array is full
 //             word 1: wgt, a, b, (k0 | k1 << 16)
-//             word 2 (inverse map only): .x the position of the sample's pair in the pair array
-//                     (sorted by first corner texel), or -1 if the array is full
 enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3 };
 
 // Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
@@ -503,8 +503,9 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                 keep = e.keep;
                 tx = make_int4(t00, t01, t10, t11);
                 if (BACKWARD) {
-                    w0 = make_float4(g.du, g.dv, __int_as_float(t00),
-                                     __int_as_float((g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0)));
+                    const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
+                    w0 = MODE == kModeFill ? make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1))
+                                           : make_float4(g.du, g.dv, __int_as_float(t00), __int_as_float(fl));
                     w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
                 } else {
                     w0 = make_float4(w00 * e.wgt, w01 * e.wgt, w10 * e.wgt, w11 * e.wgt);
@@ -560,8 +561,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                 pos = atomicAdd(cursor + i0, 1);
                 pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
             }
-            float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
-            e[ENTRY_F4 - 1] = make_float4(__int_as_float(pos), 0.f, 0.f, 0.f);
+            reinterpret_cast<int *>(L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4)[3] = pos;
         }
         if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
     }
@@ -847,7 +847,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
     const int *__restrict__ chunk_prefix, int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap) {
     extern __shared__ float4 smem[];
-    constexpr int EF4 = FILL ? 3 : 2;
+    constexpr int EF4 = 2;
+    // first corner texel and clamp flags of an entry
+    auto entry_texel = [](const float4 &geo) { return FILL ? __float_as_int(geo.z) >> 2 : __float_as_int(geo.z); };
+    auto entry_flags = [](const float4 &geo) { return FILL ? __float_as_int(geo.z) & 3 : __float_as_int(geo.w); };
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
@@ -937,14 +940,14 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 const float wgt = my[EF4 * e + 1].x;
                 const float du = geo.x, dv = geo.y;
                 const float w00 = (1.0f - du) * (1.0f - dv), w01 = (1.0f - du) * dv, w10 = du * (1.0f - dv), w11 = du * dv;
-                const int t00 = __float_as_int(geo.z), fl = __float_as_int(geo.w);
+                const int t00 = entry_texel(geo), fl = entry_flags(geo);
                 const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
                 // feature rows in address units: one 32-bit multiply and three adds, then a shift-add each
                 const unsigned r00 = (unsigned)t00 * (unsigned)k.row_units;
                 const unsigned r01 = r00 + ((fl & 2) ? row_step_v : 0u);
                 const unsigned r10 = r00 + ((fl & 1) ? (unsigned)k.row_units : 0u), r11 = r01 + (r10 - r00);
                 // scatter path, or a sample without room in the pair array: atomics for all four corners
-                const bool spill = FILL ? __float_as_int(my[EF4 * e + 2].x) < 0 : true;
+                const bool spill = FILL ? __float_as_int(geo.w) < 0 : true;
                 const bool s00 = spill, s01 = spill, s10 = spill, s11 = spill;
                 const float a00 = w00 * wgt, a01 = w01 * wgt, a10 = w10 * wgt, a11 = w11 * wgt;
 #pragma unroll
@@ -991,7 +994,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                     const float4 geo = my[EF4 * e], dw = my[EF4 * e + 1];
                     const float du = geo.x, dv = geo.y;
                     const float wc[4] = {(1.0f - du) * (1.0f - dv), (1.0f - du) * dv, du * (1.0f - dv), du * dv};
-                    const int t00 = __float_as_int(geo.z), fl = __float_as_int(geo.w);
+                    const int t00 = entry_texel(geo), fl = entry_flags(geo);
                     const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
                     const int t[4] = {t00, t00 + sv, t00 + su, t00 + sv + su};
                     const int kk = __float_as_int(dw.w);
@@ -1051,7 +1054,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                     const float4 *lst_s = my;
                     for (int pe = lis; pe < n; pe += k.lanes_per_slot) {
                         const float4 geo = lst_s[EF4 * pe], dwp = lst_s[EF4 * pe + 1];
-                        const int posp = __float_as_int(lst_s[EF4 * pe + 2].x);
+                        const int posp = __float_as_int(geo.w);
                         const int kk = __float_as_int(dwp.w);
                         const int k0 = parametric ? 0 : (kk & 0xffff), k1 = parametric ? 1 : (kk >> 16);
                         // G * a and G * b (G already carries 1/count)
@@ -1060,15 +1063,15 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                             const int word = fold ? ((pcell << k.bin_bits) | k0) : pcell;
                             float4 *dst = reinterpret_cast<float4 *>(pairs + posp);
                             dst[0] = make_float4(__int_as_float(word), dwp.x * pinv, geo.x, geo.y);
-                            dst[1] = make_float4(ga, gb, geo.w, 0.0f);
+                            dst[1] = make_float4(ga, gb, __int_as_float(entry_flags(geo)), 0.0f);
                         } else if (fold) {
                             const float du = geo.x, dv = geo.y;
-                            const int fl = __float_as_int(geo.w);
+                            const int fl = entry_flags(geo), t00 = entry_texel(geo);
 #pragma unroll
                             for (int c = 0; c < 4; ++c) {
                                 // corner c: 0 (v0,u0) 1 (v1,u0) 2 (v0,u1) 3 (v1,u1); same products as phase A
                                 const float wcc = ((c & 2) ? du : 1.0f - du) * ((c & 1) ? dv : 1.0f - dv);
-                                const int tt = __float_as_int(geo.z) + ((c & 1) && (fl & 2) ? k.W : 0) + ((c & 2) ? (fl & 1) : 0);
+                                const int tt = t00 + ((c & 1) && (fl & 2) ? k.W : 0) + ((c & 2) ? (fl & 1) : 0);
                                 atomic_add_f32(d_depth + (size_t)tt * Dd + k0, ga * wcc);
                                 atomic_add_f32(d_depth + (size_t)tt * Dd + k1, gb * wcc);
                             }
@@ -1968,7 +1971,8 @@ int validate(const fbev_problem *p, bool need_channels) {
 }
 
 int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWavesPerBlock, int max_rounds = 8,
-              int entry_bytes = 48 + 4, int slot_budget = kMaxSlotLdsBytes) {
+              int slot_budget = kMaxSlotLdsBytes) {
+    const int entry_bytes = 32 + 4;      // an entry (two float4 in every kernel) and its candidate index
     KParams &k = plan->k;
     k.B = p->batch; k.N = p->num_cams; k.H = p->feat_h; k.W = p->feat_w; k.C = p->channels;
     k.gx = p->grid_x; k.gy = p->grid_y; k.gz = p->grid_z;
@@ -2008,8 +2012,7 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     plan->cpl = cpl;
     k.lanes_per_slot = lps;
     int slots = kWave / lps;
-    // the lists must fit the per-wave LDS budget (entry_bytes per sample: the entry, up to three
-    // float4 in the backward, and the candidate index)
+    // the lists must fit the per-wave LDS budget
     while (slots > 1 && (long long)slots * k.NZ * entry_bytes > slot_budget) --slots;
     if (slots > 16) slots = 16;
     k.slots = slots;
@@ -2039,7 +2042,7 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     }
     plan->lds_fwd = block_lds(2);
     plan->lds_bwd = block_lds(2);
-    plan->lds_fill = block_lds(3);
+    plan->lds_fill = block_lds(2);
     plan->lds_count = block_lds(0);
     if (plan->lds_fill > (size_t)kLdsLimitBytes) return FBEV_ERR_TOO_LARGE;
     return FBEV_OK;
@@ -2199,11 +2202,9 @@ int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, co
     Plan pl;
     // 128-bit gathers and stores need 16-byte aligned feature and result tensors
     // measured: the forward is fastest with at most 4 rounds per wavefront, the backward's cell pass with 8
-    // Its entries are two float4, and more cells per round pay for the LDS (measured with 64 channels on a
-    // 400x400 grid: 12 height bins 115 -> 94 us with four cells per round instead of three; 20 bins 223 -> 166 us,
-    // 40 bins 785 -> 476 us); the cell pass of the backward is better off with the smaller budget.
-    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kWavesPerBlock, 4, 32 + 4,
-                   kForwardSlotLdsBytes);
+    // More cells per round pay for the LDS here (measured with 64 channels on a 400x400 grid: 20 height bins
+    // 185 -> 166 us, 40 bins 785 -> 476 us); the cell pass of the backward is better off with the smaller budget.
+    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kWavesPerBlock, 4, kForwardSlotLdsBytes);
     if (rc != FBEV_OK) return rc;
     return dispatch_forward(p, pl, depth, feats, proj, out, count_out, static_cast<hipStream_t>(stream));
 }
