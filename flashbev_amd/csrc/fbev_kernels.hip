@@ -520,7 +520,8 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         // shuffles cost the cell pass more than the saved returning atomics.)
         if (MODE == kModeCount) {
             const int prev_keep = __shfl_up((int)keep, 1, kWave);
-            const bool cont = keep && lane > 0 && prev_keep != 0 && prev_slot == slot && __shfl_up(tx.x, 1, kWave) == tx.x;
+            const int prev_texel = __shfl_up(tx.x, 1, kWave);      // every lane takes part in the exchange
+            const bool cont = keep && lane > 0 && prev_keep != 0 && prev_slot == slot && prev_texel == tx.x;
             const unsigned long long cm = __ballot(cont);
             // first lane of my run: the highest lane at or below me that does not continue
             const int run_lead = 63 - __clzll(~cm & lanemask_le(lane));

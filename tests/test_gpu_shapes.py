@@ -302,3 +302,24 @@ def test_projection_kernel_against_the_closed_form_in_float64():
         assert torch.allclose(create_projection_matrix(*args), out.cpu(), rtol=1e-4, atol=1e-3)
     assert capi.projection_matrices(0, 0, 0, 0, 0, 0) == 0          # nothing to do
     assert capi.projection_matrices(0, 0, 0, 0, 0, 4) == -1         # NULL pointers
+
+
+@pytest.mark.parametrize("feat_hw", [(1, 1), (1, 7), (5, 1), (2, 2), (3, 5), (16, 44)])
+@pytest.mark.parametrize("dist", [1, 2])
+def test_tiny_feature_maps_and_clamped_corners(feat_hw, dist):
+    """Feature maps of one row, one column or one texel: every sample's second corner is clamped
+    onto the first (u1 == u0 and / or v1 == v0), and a texel has no left or upper neighbour whose
+    samples could reach it.  The inverse map files a sample under its first corner and the texel
+    pass reads the neighbours' lists, so these are its edge cases; threshold 0 keeps every sample
+    in view, including those in the last column and row."""
+    w = small("cfg1_tiny", channels=16, feat_hw=feat_hw, grid_size=(24, 24, 4), depth_bins=16)
+    x = make_inputs(w, MODEL[dist], device="cuda", with_grad_out=True)
+    geo = c_oracle.geometry(x["projection_matrices"].cpu().numpy(), w.feat_hw, w.image_hw, list(w.roi_range),
+                            list(w.grid_size))
+    valid = geo["mask"].astype(bool)
+    assert valid.sum() > 50
+    if feat_hw[1] > 1:
+        idx = geo["idx"][valid]
+        assert (idx[:, 0] == idx[:, 1]).any() or feat_hw == (16, 44)      # some u1 clamped onto u0
+    print(f"[case] feat_hw={feat_hw} dist={dist} valid={int(valid.sum())}", flush=True)
+    check_all(w, x, dist, thr=0.0, modes=("scatter", "gather", "gather_overwrite", "gather_counted", "columns"))
