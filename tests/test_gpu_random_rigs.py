@@ -36,7 +36,7 @@ def random_pose(rng):
     return (K4 @ np.linalg.inv(T))[:3]
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(20))
 def test_random_rig(seed):
     rng = np.random.default_rng(100 + seed)
     n_cams = int(rng.integers(1, 5))
