@@ -323,3 +323,19 @@ def test_tiny_feature_maps_and_clamped_corners(feat_hw, dist):
         assert (idx[:, 0] == idx[:, 1]).any() or feat_hw == (16, 44)      # some u1 clamped onto u0
     print(f"[case] feat_hw={feat_hw} dist={dist} valid={int(valid.sum())}", flush=True)
     check_all(w, x, dist, thr=0.0, modes=("scatter", "gather", "gather_overwrite", "gather_counted", "columns"))
+
+
+def test_long_sample_lists_need_more_than_64_kib_of_lds():
+    """6 cameras x 100 height bins = 600 samples per cell: the forward's lists take more than the
+    64 KiB of dynamic LDS a kernel gets without asking; far beyond that the library refuses."""
+    w = small(channels=8, grid_size=(8, 8, 100))
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    print("[case] long lists NZ=600", flush=True)
+    check_all(w, x, 1, thr=0.0, modes=("scatter", "gather", "gather_counted"))
+    w = small(channels=8, grid_size=(8, 8, 400))
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    p = U.problem_for(x, w, 1)
+    out = torch.empty((1, 8, 8, 8), dtype=torch.float32, device="cuda")
+    rc = capi.forward(p, x["depth_params"].data_ptr(), x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(),
+                      out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == -4 and "too large" in capi.status_string(rc)
