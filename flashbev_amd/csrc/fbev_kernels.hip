@@ -1099,8 +1099,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
 constexpr int kTexelMaxSplit = 8;
 constexpr int kTexelSplitBelow = 8192;
 constexpr int kTexelPart = 128;
-constexpr int kTexelNarrowFrom = 50000;
-constexpr int kTexelNarrowPairs = 512;       // upper bound of samples per list
+constexpr int kTexelOneWaveBelow = 100;      // possible samples per texel below which a block is one wavefront ...
+constexpr int kTexelManyTexels = 50000;      // ... or three times that when there are this many texels
+constexpr int kTexelTwoWavesBelow = 450;     // below which it is two wavefronts; four from there on
 constexpr int kTexelSegs = 4 * kFixedReplicas;   // lists of a texel with fixed segments: 4 first corners x replicas
 template <int VEC, int WAVES>
 __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
@@ -2363,11 +2364,16 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const int vec = vec4 ? 4 : 1;
     const int cq = (p->channels + vec - 1) / vec;
     const int lpr = cq < kWave ? cq : kWave;
-    // Four wavefronts per texel, or one (taking the four segments in turn) when there are many
-    // texels whose lists cannot be long: measured at 67 584 texels reached by about 57 sample corners
-    // each, one wavefront is 24 % faster than four; at 33 792 texels with about 280, two are 18 % slower.
-    const bool short_lists = texels >= kTexelNarrowFrom && fbev_backward_max_pairs(p) / (uint64_t)texels < kTexelNarrowPairs;
-    const int texel_waves = short_lists ? 1 : kWavesPerBlock;
+    // One, two or four wavefronts per texel.  A texel's block is a chain of dependent loads (list bounds,
+    // pairs, grad_out rows); small blocks fit the machine in fewer generations, large ones shorten the
+    // chain of a long list.  What is known here is only how many samples a texel could get if every one were
+    // kept.  Measured (us for 1 / 2 / 4 wavefronts; Laplace, then the categorical model, which keeps twice
+    // as many): 23 possible samples per texel 8 / 9 / 11; 186 per texel and 4224 texels 20 / 19 / 23 and
+    // 39 / 30 / 31; 186 per texel and 67 584 texels 125 / 154 / 239 and 256 / 274 / 365; 454 per texel
+    // 38 / 29 / 29 and 80 / 60 / 52; 909 per texel 493 / 426 / 431; 2727 per texel 352 / 209 / 124.
+    const uint64_t per_texel = fbev_backward_max_pairs(p) / (uint64_t)texels;
+    const int texel_waves = (per_texel < kTexelOneWaveBelow || (texels >= kTexelManyTexels && per_texel < 3 * kTexelOneWaveBelow)) ? 1
+                            : (per_texel < kTexelTwoWavesBelow ? 2 : kWavesPerBlock);
     const int nw = (kWave / lpr) * texel_waves;
     // the depth gradient rides on the pairs exactly when the cell pass folds it in (one channel pass
     // and room for the depth bin in a pair's first word)
@@ -2379,18 +2385,19 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);
     const dim3 tgrid((unsigned)texels, n_split), tblock(kWave * texel_waves);
-    if (vec4 && short_lists)
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<4, 1>), tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor,
-                           pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
-    else if (vec4)
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<4, kWavesPerBlock>), tgrid, tblock, lds, st, pl.k, grad_out,
-                           prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
-    else if (short_lists)
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<1, 1>), tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor,
-                           pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
-    else
-        hipLaunchKernelGGL((fbev_backward_texel_kernel<1, kWavesPerBlock>), tgrid, tblock, lds, st, pl.k, grad_out,
-                           prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats, lpr, from_pairs);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats,
+                           lpr, from_pairs);
+    };
+    if (vec4) {
+        if (texel_waves == 1) launch(fbev_backward_texel_kernel<4, 1>);
+        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<4, 2>);
+        else launch(fbev_backward_texel_kernel<4, kWavesPerBlock>);
+    } else {
+        if (texel_waves == 1) launch(fbev_backward_texel_kernel<1, 1>);
+        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<1, 2>);
+        else launch(fbev_backward_texel_kernel<1, kWavesPerBlock>);
+    }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 

