@@ -82,16 +82,15 @@ constexpr int kForwardSlotLdsBytes = 20000;  // the same for the forward kernel
 constexpr int kMaxBlockLdsBytes = 64 * 1024; // dynamic LDS a block may ask for without opting in
 constexpr int kLdsLimitBytes = 150 * 1024;   // what a block may ask for at all (160 KiB per CU)
 constexpr int kXcdCount = 8;                 // accelerator complex dies, each with its own L2
-// The inverse map counts sample corners per texel with integer atomics.  Atomics on one
-// address execute one after the other, and the texels on the horizon collect thousands of
+// The inverse map counts the samples per first-corner texel with integer atomics.  Atomics on
+// one address execute one after the other, and the texels on the horizon collect thousands of
 // samples, so every texel owns kReplicas counters and a sample picks one from its cell.
 constexpr int kReplicaBits = 5;
 constexpr int kReplicas = 1 << kReplicaBits;
-// With fixed-capacity segments (no counting pass) a texel has one segment per wavefront of the
-// block that later gathers it.
+// With fixed-capacity segments (no counting pass) a texel has four segments, again chosen by cell.
 constexpr int kFixedReplicas = 4;
 constexpr int kFixedMinSegment = 4;           // shorter segments would mostly overflow: count instead
-static_assert(kFixedReplicas == 4, "the texel pass reads a texel's claim counters as one int4");
+static_assert(kFixedReplicas == 4, "the texel pass numbers a texel's lists first corner + 4 * replica");
 constexpr int kScanChunkBits = 12;           // counters are prefix-summed in chunks of 4096
 
 struct KParams {
@@ -392,7 +391,7 @@ constexpr float kEarlySlack = 1.0e-3f;
 //   stage 2  lanes = candidates, densely packed: the canonical arithmetic (divisions, floor,
 //            bilinear weights), the depth model, the weight threshold; what is kept goes, still
 //            in (camera, height) order, into its slot's entry list.
-// kModeCount writes no entries; it only counts the kept sample corners per (texel, replica).
+// kModeCount writes no entries; it only counts the kept samples per (first-corner texel, replica).
 template <int ENTRY_F4, typename T, int MODE>
 __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, const T *__restrict__ depth, int b, int q0,
                                         int lane, const int *__restrict__ chunk_prefix = nullptr,
@@ -695,9 +694,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
 // Two ways to form the feature gradient, which is a sum over all samples that touch a texel:
 //   scatter      fbev_backward_cells_kernel<.., false>: one hardware fp32 atomic per (sample,
 //                corner, channel).  Needs no workspace; slow under contention.
-//   inverse map  count the samples per texel, prefix-sum the counts, let the cell pass
-//                (fbev_backward_cells_kernel<.., true>) drop one 16-byte (cell, coefficient)
-//                pair per sample corner into the texel's segment, then gather per texel
+//   inverse map  let the cell pass (fbev_backward_cells_kernel<.., true>) drop one 32-byte record
+//                per kept sample into the segment of the sample's first corner texel (segments
+//                of fixed capacity, or packed after a counting pass and a prefix sum), then
+//                gather per texel from the segments of the four texels whose samples reach it
 //                (fbev_backward_texel_kernel): the same coalesced row reads as the forward
 //                pass, no floating-point atomics, each gradient row written once.
 __device__ __forceinline__ void atomic_add_f32(float *p, float v) { unsafeAtomicAdd(p, v); }
@@ -743,7 +743,7 @@ __global__ __launch_bounds__(256) void fbev_fill_zero_kernel(int *a, long long n
     else if (i < ua + ub + uc) zero_unit(c, nc, i - ua - ub);
 }
 
-// Count, per (texel, replica), the sample corners that will contribute: phase A alone, with
+// Count, per (first-corner texel, replica), the samples that will contribute: phase A alone, with
 // exactly the decisions the cell pass takes later (same code, same inputs).
 template <typename T>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_count_kernel(KParams k, const T *__restrict__ depth,
@@ -2307,7 +2307,7 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     if ((uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
     const size_t index_bytes = ws_index_bytes(p);
     if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
-    // pair positions are 32-bit: every sample corner must be countable
+    // pair positions are 32-bit: every sample must be countable
     if (sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
     // the texel pass addresses grad_out rows in 32-bit units (16 bytes, or one float off the vector path)
     const bool rows_vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
@@ -2325,7 +2325,7 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const long long counters = counter_count(p), chunks = chunk_count(p);
     int *chunk_prefix = cursor + counters;
 
-    // A workspace with room for every sample corner gets fixed segments: each (texel, replica)
+    // A workspace with room for every sample gets fixed segments: each (texel, replica)
     // owns cap / (texels * kFixedReplicas) pair slots, and the counting pass and the prefix sums
     // are not needed.  (A texel that outgrows its segments falls back to atomics, like a full
     // pair array does.)  Smaller workspaces are packed exactly: count, scan, fill.

@@ -234,7 +234,7 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                                      ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, st);
     };
     // Inverse-map gather.  The pair array comes from PyTorch's caching allocator (no device
-    // allocation in steady state).  By default it has room for every sample corner, which lets
+    // allocation in steady state).  By default it has room for every sample, which lets
     // the library use fixed per-texel segments and skip its counting pass; a smaller
     // pair_capacity selects the exactly packed layout (what does not fit is applied with atomics).
     auto run_gather = [&]() -> int {
