@@ -1107,7 +1107,7 @@ template <int VEC, int WAVES>
 __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
     const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
-    float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs) {
+    float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs, int fresh) {
     extern __shared__ float4 smem[];
     float *part = reinterpret_cast<float *>(smem);
     // Blocks are dealt to the accelerator dies in turn; let each die walk a contiguous range of
@@ -1135,6 +1135,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     // e): no LDS, no barrier before the first pair is requested.
     const int tu = t % k.W, tv = (t / k.W) % k.H;
     int my_lo = 0, my_len = 0;
+    bool spilled = false;      // a list of this texel was full: the cell pass added the rest with atomics
     if (lane < kTexelSegs) {
         const int e = lane;
         const int o = counted ? e : e & 3;
@@ -1145,12 +1146,16 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             // replica to the end of this texel's
             const long long first = (long long)q * kReplicas - 1, last = (long long)q * kReplicas + kReplicas - 1;
             my_lo = q == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
-            my_len = max(min(chunk_prefix[last >> kScanChunkBits] + seg_end[last], pair_cap) - my_lo, 0);
+            const int list_end = chunk_prefix[last >> kScanChunkBits] + seg_end[last];
+            spilled = list_end > pair_cap;
+            my_len = max(min(list_end, pair_cap) - my_lo, 0);
         } else if (exists) {
             // fixed segments of pair_cap pairs; seg_end holds how many were claimed
             const int i = q * kFixedReplicas + (e >> 2);
             my_lo = i * pair_cap;
-            my_len = max(min(seg_end[i], pair_cap), 0);
+            const int claimed = seg_end[i];
+            spilled = claimed > pair_cap;
+            my_len = max(min(claimed, pair_cap), 0);
         }
     }
     // the lists one after the other form one sequence of pairs; list e starts at my_pre of lane e
@@ -1168,6 +1173,10 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     const int n_parts = min((int)gridDim.y, (n_all + 4 * kTexelPart - 1) / (4 * kTexelPart));
     if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
     const bool shared_texel = n_parts > 1;
+    // The gradient buffers were cleared by this call (fresh) and nothing but this block touches the
+    // texel unless a list spilled: then its rows are stored, not added, and the pass ends without a
+    // dependent load.
+    const bool store_only = fresh != 0 && !shared_texel && __ballot(spilled) == 0ull;
     const int part_lo = (int)(((long long)n_all * blockIdx.y) / n_parts);
     const int part_hi = (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
     // the wavefronts take chunks of the sequence in turn: 64 pairs, fewer when that leaves a wavefront idle
@@ -1305,6 +1314,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             if (d_feats != nullptr) {
                 float *dst = d_feats + (size_t)t * k.C + c0 + c;
                 if (shared_texel) atomic_add_f32(dst, sum);
+                else if (store_only) *dst = sum;
                 else *dst += sum;
             }
         }
@@ -1314,6 +1324,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
                 if (sum != 0.0f) {
                     float *dst = d_depth + (size_t)t * k.Dd + i;
                     if (shared_texel) atomic_add_f32(dst, sum);
+                    else if (store_only) *dst = sum;
                     else *dst += sum;
                 }
             }
@@ -1322,6 +1333,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             for (int w = 0; w < nw; ++w) sum += part[w * stride + span + threadIdx.x];
             float *dst = d_depth + (size_t)t * 2 + threadIdx.x;
             if (shared_texel) atomic_add_f32(dst, sum);
+            else if (store_only) *dst = sum;
             else *dst += sum;
         }
     }
@@ -2387,7 +2399,7 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     const dim3 tgrid((unsigned)texels, n_split), tblock(kWave * texel_waves);
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats,
-                           lpr, from_pairs);
+                           lpr, from_pairs, accumulate ? 0 : 1);
     };
     if (vec4) {
         if (texel_waves == 1) launch(fbev_backward_texel_kernel<4, 1>);
