@@ -90,6 +90,7 @@ constexpr int kReplicas = 1 << kReplicaBits;
 // With fixed-capacity segments (no counting pass) a texel has four segments, again chosen by cell.
 constexpr int kFixedReplicas = 4;
 constexpr int kFixedMinSegment = 4;           // shorter segments would mostly overflow: count instead
+constexpr int kClaimRunsFrom = 300;           // possible samples per claim counter from which runs claim together
 static_assert(kFixedReplicas == 4, "the texel pass numbers a texel's lists first corner + 4 * replica");
 constexpr int kScanChunkBits = 12;           // counters are prefix-summed in chunks of 4096
 
@@ -102,7 +103,8 @@ struct KParams {
     int blocks_per_batch;
     int slots;           // S: cells per wavefront per round
     int rounds;          // rounds per wavefront
-    int lanes_per_slot;  // lanes that carry channels in phase B
+    int lanes_per_slot;  // lanes that carry channels in phase B (one lane group)
+    int groups_per_slot; // lane groups that share a slot's list (more than one when long lists leave few slots)
     int list_cap;        // entries per slot list (= NZ)
     float Wi_f, Hi_f, W_f, H_f;
     float xmin, ymin, zmin, vx, vy, vz;
@@ -371,7 +373,7 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 //                     the two flags below it, and in the fourth place the position of the sample's
 //                     pair in the pair array (sorted by first corner texel), or -1 if the array is full
 //             word 1: wgt, a, b, (k0 | k1 << 16)
-enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3 };
+enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeFillRuns = 4 };
 
 // Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
 // pixel coordinate misses the image by more than this fraction, far beyond any rounding of
@@ -396,7 +398,8 @@ template <int ENTRY_F4, typename T, int MODE>
 __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, const T *__restrict__ depth, int b, int q0,
                                         int lane, const int *__restrict__ chunk_prefix = nullptr,
                                         int *__restrict__ cursor = nullptr, int pair_cap = 0) {
-    constexpr bool BACKWARD = MODE == kModeScatter || MODE == kModeFill;
+    constexpr bool FILLING = MODE == kModeFill || MODE == kModeFillRuns;   // the latter claims per run
+    constexpr bool BACKWARD = MODE == kModeScatter || FILLING;
     const int n_cols = k.slots * k.N;
     if (lane < 16) L.cnt[lane] = 0;
     if (lane < k.slots) {
@@ -503,7 +506,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                 tx = make_int4(t00, t01, t10, t11);
                 if (BACKWARD) {
                     const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
-                    w0 = MODE == kModeFill ? make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1))
+                    w0 = FILLING ? make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1))
                                            : make_float4(g.du, g.dv, __int_as_float(t00), __int_as_float(fl));
                     w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
                 } else {
@@ -515,18 +518,23 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         // Consecutive height bins of one (cell, camera) often fall on the same texel (far cells
         // compress onto the horizon rows).  Samples that repeat the first corner of the previous
         // kept sample of the same cell form a run; when counting, the run's first lane adds the
-        // whole run with ONE atomic.  (Claiming positions per run as well was measured: the
-        // shuffles cost the cell pass more than the saved returning atomics.)
-        if (MODE == kModeCount) {
+        // whole run with ONE atomic.  Positions are claimed per run as well where a claim counter
+        // may get hundreds of samples (kModeFillRuns): claims on one address are served one
+        // after the other, and a 400 x 400 x 12 grid on 4224 texels spent half of the cell pass
+        // waiting for them.  Elsewhere the shuffles cost more than the saved returning atomics.
+        int run_lead = lane, run_len = 1;
+        if (MODE == kModeCount || MODE == kModeFillRuns) {
             const int prev_keep = __shfl_up((int)keep, 1, kWave);
             const int prev_texel = __shfl_up(tx.x, 1, kWave);      // every lane takes part in the exchange
             const bool cont = keep && lane > 0 && prev_keep != 0 && prev_slot == slot && prev_texel == tx.x;
             const unsigned long long cm = __ballot(cont);
             // first lane of my run: the highest lane at or below me that does not continue
-            const int run_lead = 63 - __clzll(~cm & lanemask_le(lane));
+            run_lead = 63 - __clzll(~cm & lanemask_le(lane));
             // lanes after me that continue without a gap
             const unsigned long long after = lane == 63 ? 0ull : (cm >> (lane + 1));
-            const int run_len = 1 + (~after == 0ull ? 63 - lane : __ffsll((long long)~after) - 1);
+            run_len = 1 + (~after == 0ull ? 63 - lane : __ffsll((long long)~after) - 1);
+        }
+        if (MODE == kModeCount) {
             if (keep && run_lead == lane)
                 atomicAdd(cursor + tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16), run_len);
             continue;
@@ -563,6 +571,25 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
             }
             reinterpret_cast<int *>(L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4)[3] = pos;
         }
+        if (MODE == kModeFillRuns) {
+            // the same, but the run's first lane claims for the whole run (same cell and texel: same
+            // counter) and hands the positions out; every lane takes part in the exchange
+            const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
+            const bool counted = chunk_prefix != nullptr;
+            const int i0 = counted ? tx.x * kReplicas + rep : tx.x * kFixedReplicas + (rep & (kFixedReplicas - 1));
+            int pos = 0;
+            if (keep && run_lead == lane) pos = atomicAdd(cursor + i0, run_len);
+            pos = __shfl(pos, run_lead, kWave) + (lane - run_lead);
+            if (keep) {
+                if (counted) {
+                    pos += chunk_prefix[i0 >> kScanChunkBits];
+                    pos = pos < pair_cap ? pos : -1;
+                } else {
+                    pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
+                }
+                reinterpret_cast<int *>(L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4)[3] = pos;
+            }
+        }
         if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
     }
 }
@@ -584,8 +611,12 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     float4 *lst = L.lst;
 
     const int cells_per_wave = k.slots * k.rounds;
-    const int slot = lane / k.lanes_per_slot;
-    const int lis = lane - slot * k.lanes_per_slot;
+    // a lane group covers the channels of one cell; when long lists leave room for few slots,
+    // several groups share a slot and take its entries in turn
+    const int gps = k.groups_per_slot;
+    const int group = lane / k.lanes_per_slot;
+    const int slot = group / gps, sub = group - slot * gps;
+    const int lis = lane - group * k.lanes_per_slot;
     const bool carrier = slot < k.slots;
     const int span = k.lanes_per_slot * VEC * CPL;   // channels covered per pass
     constexpr int kUnitShift = VEC > 1 ? 4 : (sizeof(T) == 4 ? 2 : 1);
@@ -605,7 +636,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
         const int n = mine ? cnt[slot] : 0;
         const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * 2;
         // the number of samples that enter the mean; the backward pass can reuse it
-        if (count_out != nullptr && mine && lis == 0) count_out[((size_t)b * k.gy + iy) * k.gx + ix] = (float)n;
+        if (count_out != nullptr && mine && lis == 0 && sub == 0) count_out[((size_t)b * k.gy + iy) * k.gx + ix] = (float)n;
         float *o = out + (((size_t)b * k.gy + iy) * k.gx + ix) * k.C;
         for (int c0 = 0; out != nullptr && c0 < k.C; c0 += span) {
             float acc[CPL][VEC];
@@ -644,10 +675,11 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
             };
             // two entries per trip where the registers allow, all eight row loads issued before the
             // first is used (the loop is a chain of gather latencies, not of arithmetic)
-            int e = 0;
+            // (group `sub` of the slot takes the entry pairs sub, sub + gps, ...)
             if (CPL == 1) {
                 const int ch = c0 + lis * VEC;
-                for (; ch < k.C && e + 1 < n; e += 2) {
+                int e = 2 * sub;
+                for (; ch < k.C && e + 1 < n; e += 2 * gps) {
                     const float4 wa = my[2 * e], ta = my[2 * e + 1], wb = my[2 * e + 2], tb = my[2 * e + 3];
                     const int off[8] = {__float_as_int(ta.x), __float_as_int(ta.y), __float_as_int(ta.z), __float_as_int(ta.w),
                                         __float_as_int(tb.x), __float_as_int(tb.y), __float_as_int(tb.z), __float_as_int(tb.w)};
@@ -661,9 +693,23 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
 #pragma unroll
                         for (int v = 0; v < VEC; ++v) acc[0][v] = __builtin_fmaf(wv[c], f[c][v], acc[0][v]);
                 }
+                if (e < n) gather(e);       // the odd entry at the end falls to one group
+            } else {
+                for (int e = sub; e < n; e += gps) gather(e);
             }
-            for (; e < n; ++e) gather(e);
-            if (mine) {
+            // the groups of a slot add up in its first group
+            if (gps > 1) {
+#pragma unroll
+                for (int jj = 0; jj < CPL; ++jj)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        const float part = acc[jj][v];
+                        float sum = part;
+                        for (int j = 1; j < gps; ++j) sum += __shfl_down(part, j * k.lanes_per_slot, kWave);
+                        acc[jj][v] = sum;
+                    }
+            }
+            if (mine && sub == 0) {
                 // the mean as a product with 1/n (one division per cell instead of one per channel;
                 // it can differ from the quotient in the last place)
                 const float scale = k.reduce_sum ? 1.0f : (n > 0 ? 1.0f / (float)n : 0.0f);
@@ -839,10 +885,11 @@ __global__ __launch_bounds__(1024) void fbev_scan_sums_kernel(int *v, int n) {
     }
 }
 
-// Cell pass of the backward.  FILL = false: scatter with atomics.  FILL = true: write pairs.
+// Cell pass of the backward.  FILL = 0: scatter with atomics.  FILL = 1: write pairs (inverse
+// map); FILL = 2: the same with one claim per run of samples on one texel.
 // `cursor` holds, on entry, the start (within its scan chunk) of every (texel, replica)
 // segment; phase A advances it, so on exit cursor[i] is the END of segment i.
-template <typename T, int VEC, int CPL, bool FILL>
+template <typename T, int VEC, int CPL, int FILL>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_kernel(
     KParams k, const float *__restrict__ grad_out, const T *__restrict__ depth, const T *__restrict__ feats,
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
@@ -863,8 +910,11 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     float4 *lst = L.lst;
 
     const int cells_per_wave = k.slots * k.rounds;
-    const int slot = lane / k.lanes_per_slot;
-    const int lis = lane - slot * k.lanes_per_slot;
+    // lane groups of lanes_per_slot lanes; the groups_per_slot groups of a slot take its entries in turn
+    const int gps = k.groups_per_slot;
+    const int group = lane / k.lanes_per_slot;
+    const int slot = group / gps, sub = group - slot * gps;
+    const int lis = lane - group * k.lanes_per_slot;
     const bool carrier = slot < k.slots;
     const int span = k.lanes_per_slot * VEC * CPL;
     const int Dd = k.Dd;
@@ -875,6 +925,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     // G of four entries is summed over the lanes of a slot at a time when the slots start on
     // multiples of four lanes (always, on the 128-bit path)
     const bool grouped = (k.lanes_per_slot & 3) == 0;
+    // first step of the sum over a slot's lanes: the largest power of two below the slot's width
+    int red_first = 32;
+    while (red_first >= k.lanes_per_slot && red_first > 1) red_first >>= 1;
     // The depth gradient travels with the pairs when one channel pass sees the whole of G and
     // the pair's first word has room for the depth bin; otherwise it is added with atomics here.
     const bool fold = FILL && need_G && k.C <= span && k.bin_bits >= 0;
@@ -912,7 +965,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
             }
         };
         load_g(0);
-        phase_a<EF4, T, FILL ? kModeFill : kModeScatter>(k, L, depth, b, q0, lane, chunk_prefix, cursor, pair_cap);
+        phase_a<EF4, T, FILL == 2 ? kModeFillRuns : (FILL ? kModeFill : kModeScatter)>(k, L, depth, b, q0, lane, chunk_prefix, cursor, pair_cap);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 
@@ -1010,7 +1063,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
             };
 
             if (grouped) {
-                for (int e0 = 0; e0 < n_max; e0 += 4) {
+                for (int t0 = 0; t0 < n_max; t0 += 4 * gps) {
+                    const int e0 = t0 + 4 * sub;
                     float G0 = e0 < n ? entry_share(e0) : 0.0f;
                     float G1 = e0 + 1 < n ? entry_share(e0 + 1) : 0.0f;
                     float G2 = e0 + 2 < n ? entry_share(e0 + 2) : 0.0f;
@@ -1023,8 +1077,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                         const float ka = (b0 ? G2 : G0) + ra, kb = (b0 ? G3 : G1) + rb;
                         float Gq = (b1 ? kb : ka) + quad_xor2(b1 ? ka : kb);
                         // ... and four more add up the groups of the slot
-#pragma unroll
-                        for (int off = 32; off >= 4; off >>= 1) {
+                        for (int off = red_first; off >= 4; off >>= 1) {
                             const float other = __shfl_down(Gq, off, kWave);
                             if (lis + off < k.lanes_per_slot) Gq += other;
                         }
@@ -1033,11 +1086,11 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                     }
                 }
             } else {
-                for (int e = 0; e < n_max; ++e) {
+                for (int t0 = 0; t0 < n_max; t0 += gps) {
+                    const int e = t0 + sub;
                     float G = e < n ? entry_share(e) : 0.0f;
                     if (need_G) {
-#pragma unroll
-                        for (int off = 32; off > 0; off >>= 1) {
+                        for (int off = red_first; off > 0; off >>= 1) {
                             const float other = __shfl_down(G, off, kWave);
                             if (lis + off < k.lanes_per_slot) G += other;
                         }
@@ -1046,14 +1099,14 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 }
             }
             if (FILL && first_pass) {
-                // ---- the pairs of this round: the lanes of a slot take the slot's entries in turn
+                // ---- the pairs of this round: the lanes of a slot's groups take the slot's entries in turn
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 {
                     const int pcell = cell;
                     const float pinv = inv;
                     const float4 *lst_s = my;
-                    for (int pe = lis; pe < n; pe += k.lanes_per_slot) {
+                    for (int pe = sub * k.lanes_per_slot + lis; pe < n; pe += gps * k.lanes_per_slot) {
                         const float4 geo = lst_s[EF4 * pe], dwp = lst_s[EF4 * pe + 1];
                         const int posp = __float_as_int(geo.w);
                         const int kk = __float_as_int(dwp.w);
@@ -2031,6 +2084,7 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     while (slots > 1 && (long long)slots * k.NZ * entry_bytes > slot_budget) --slots;
     if (slots > 16) slots = 16;
     k.slots = slots;
+    k.groups_per_slot = (kWave / lps) / slots;     // >= 1: slots <= kWave / lps
     k.list_cap = k.NZ;
     // enough wavefronts to fill 256 CUs several times over before a wavefront takes more rounds
     const long long groups = ((long long)k.padded_cells + slots - 1) / slots * k.B;
@@ -2116,7 +2170,7 @@ int launch_columns(const Plan &pl, const ColParams &cp, size_t lds, const float 
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
-template <typename T, int VEC, bool FILL>
+template <typename T, int VEC, int FILL>
 int launch_cells(const Plan &pl, const float *go, const void *depth, const void *feats, const float *proj,
                  float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap, hipStream_t st) {
     dim3 grid(pl.k.n_blocks), block(kWave * pl.k.waves);
@@ -2135,7 +2189,7 @@ int launch_cells(const Plan &pl, const float *go, const void *depth, const void 
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
-template <bool FILL>
+template <int FILL>
 int dispatch_cells(const fbev_problem *p, const Plan &pl, const float *go, const void *depth, const void *feats,
                    const float *proj, float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap,
                    hipStream_t st) {
@@ -2239,7 +2293,7 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
                          static_cast<hipStream_t>(stream));
         if (rc != FBEV_OK) return rc;
     }
-    return dispatch_cells<false>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, nullptr, nullptr, nullptr, 0,
+    return dispatch_cells<0>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, nullptr, nullptr, nullptr, 0,
                                  static_cast<hipStream_t>(stream));
 }
 
@@ -2367,8 +2421,12 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     }
     const int *prefix_arg = fixed ? nullptr : chunk_prefix;
     const int cap_arg = fixed ? seg_cap : cap;
-    rc = dispatch_cells<true>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs, cap_arg,
-                              st);
+    // samples a claim counter gets if every sample is kept
+    const bool claim_runs = sample_count(p) / (fixed ? texels * kFixedReplicas : counters) >= kClaimRunsFrom;
+    rc = claim_runs ? dispatch_cells<2>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
+                                        cap_arg, st)
+                    : dispatch_cells<1>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
+                                        cap_arg, st);
     if (rc != FBEV_OK) return rc;
 
     // texel pass: rows of grad_out are fp32, so 128-bit gathers need C % 4 == 0 and aligned rows

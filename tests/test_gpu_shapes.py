@@ -328,6 +328,34 @@ def test_tiny_feature_maps_and_clamped_corners(feat_hw, dist):
     check_all(w, x, dist, thr=0.0, modes=("scatter", "gather", "gather_overwrite", "gather_counted", "columns"))
 
 
+@pytest.mark.parametrize("feat_hw", [(4, 6), (1, 2)])
+@pytest.mark.parametrize("dist", [1, 2])
+def test_many_samples_per_claim_counter_claim_by_runs(feat_hw, dist):
+    """Few texels under many samples: from 300 possible samples per claim counter on, the samples of
+    one cell that follow each other on one texel claim their pair positions with a single atomic
+    (fixed segments: 4 counters per texel; counted segments: 32, reached with the 1 x 2 map).  With
+    the default threshold some samples of a column are dropped, which breaks runs in the middle."""
+    w = small("cfg1_tiny", channels=16, feat_hw=feat_hw, grid_size=(48, 48, 16), depth_bins=16)
+    samples, texels = 48 * 48 * 16, feat_hw[0] * feat_hw[1]
+    assert samples // (texels * 4) >= 300 and (feat_hw != (1, 2) or samples // (texels * 32) >= 300)
+    x = make_inputs(w, MODEL[dist], device="cuda", with_grad_out=True)
+    for thr in (0.0, 1e-6):
+        print(f"[case] claim runs feat_hw={feat_hw} dist={dist} thr={thr}", flush=True)
+        check_all(w, x, dist, thr=thr, modes=("gather", "gather_overwrite", "gather_counted"))
+
+
+@pytest.mark.parametrize("channels,gz,dtype", [(80, 50, torch.float32), (64, 40, torch.float32),
+                                               (128, 40, torch.float16), (20, 60, torch.float32)])
+def test_lane_groups_share_the_list_of_a_cell(channels, gz, dtype):
+    """Lists of 240 to 360 samples per cell leave LDS for one or two cells per wavefront; the lane
+    groups that would otherwise idle (three of 20 lanes at 80 channels, four of 16 at 64, three of
+    five at 20) take the entries of the same cell in turn and their partial sums are added up."""
+    w = small(channels=channels, grid_size=(16, 16, gz), dtype=dtype)
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    print(f"[case] shared lists C={channels} gz={gz} {dtype}", flush=True)
+    check_all(w, x, 1, thr=0.0, modes=("scatter", "gather", "gather_counted"))
+
+
 def test_long_sample_lists_need_more_than_64_kib_of_lds():
     """6 cameras x 100 height bins = 600 samples per cell: the forward's lists take more than the
     64 KiB of dynamic LDS a kernel gets without asking; far beyond that the library refuses."""
