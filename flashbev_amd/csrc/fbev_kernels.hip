@@ -1162,7 +1162,9 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
     float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs, int fresh) {
     extern __shared__ float4 smem[];
-    float *part = reinterpret_cast<float *>(smem);
+    // per wavefront 64 (grad_out row, coefficient) records of the chunk in hand, then the partial rows
+    float2 *stage = reinterpret_cast<float2 *>(smem) + (threadIdx.x >> 6) * kWave;
+    float *part = reinterpret_cast<float *>(smem) + WAVES * kWave * 2;
     // Blocks are dealt to the accelerator dies in turn; let each die walk a contiguous range of
     // texels, column by column: the texels of a feature-map column gather the cells along one
     // wedge of rays (a cell's height bins land on neighbouring rows), so their grad_out rows meet
@@ -1263,7 +1265,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
         for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
         float sa = 0.0f, sb = 0.0f;
         // A wavefront takes 64 consecutive pairs at a time, one per lane in a single coalesced
-        // load, and hands them to its workers through lane shuffles; four grad_out rows per
+        // load, and hands them to its workers through 512 bytes of LDS; four grad_out rows per
         // worker are in flight before the first is used.  The loop is bound by load latency:
         // without this the pair load and the row load it addresses form a dependent chain.
         for (int bstart = part_lo + wave * chunk; bstart < part_hi; bstart += n_waves * chunk) {
@@ -1311,37 +1313,58 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
                     sb += pd.y * cw;
                 }
             }
-            // Full groups of UNR pairs per worker run without predicates (lanes that carry no
+            // Pairs that follow each other in a list and come from one cell (its samples on
+            // neighbouring height bins that share a first corner claimed neighbouring positions)
+            // gather the same grad_out row: their coefficients are added up and the row is
+            // gathered once.  A run gets a new leader every eight lanes, so that three steps of a
+            // suffix sum inside the runs leave every leader with its run's coefficient.
+            const unsigned prev_row = (unsigned)__shfl_up((int)my_row, 1, kWave);
+            const bool in_chunk = lane < nb;
+            const unsigned long long cm = __ballot(in_chunk && lane > 0 && my_row == prev_row);
+            const int run_lead = 63 - __clzll(~cm & lanemask_le(lane));
+            const unsigned long long lm = __ballot(in_chunk && ((lane - run_lead) & 7) == 0);
+            const unsigned long long later = lane == 63 ? 0ull : (lm >> (lane + 1));      // leaders after me
+            const int followers = later ? __ffsll((long long)later) - 1 : 63 - lane;    // lanes past the chunk carry 0
+            float run_coef = my_coef;
+#pragma unroll
+            for (int off = 1; off <= 4; off <<= 1) {
+                const float other = __shfl_down(run_coef, off, kWave);
+                if (off <= followers) run_coef += other;
+            }
+            const int n_lead = __popcll(lm);
+            if ((lm >> lane) & 1ull) stage[__popcll(lm & lanemask_lt(lane))] = make_float2(__int_as_float((int)my_row), run_coef);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            // Full groups of UNR rows per worker run without predicates (lanes that carry no
             // channel gather channel 0 of some row and drop the result); the remainder goes one
-            // pair per worker.
+            // row per worker.
             constexpr int UNR = 4;
-            const int group = wpw * UNR, full = nb - nb % group;
+            const int group = wpw * UNR, full = n_lead - n_lead % group;
             for (int i = 0; i < full; i += group) {
                 float coefs[UNR];
                 float g[UNR][VEC];
 #pragma unroll
                 for (int q = 0; q < UNR; ++q) {
-                    const int j = i + q * wpw + wslot_eff;
-                    const unsigned row = (unsigned)__shfl((int)my_row, j, kWave);
-                    coefs[q] = __shfl(my_coef, j, kWave);
-                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)row << kOutShift)) + ch_eff, g[q]);
+                    const float2 rc = stage[i + q * wpw + wslot_eff];
+                    coefs[q] = rc.y;
+                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g[q]);
                 }
 #pragma unroll
                 for (int q = 0; q < UNR; ++q)
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coefs[q], g[q][v], acc[v]);
             }
-            for (int i = full; i < nb; i += wpw) {
+            for (int i = full; i < n_lead; i += wpw) {
                 const int j = i + wslot_eff;
-                const unsigned row = (unsigned)__shfl((int)my_row, min(j, kWave - 1), kWave);
-                const float coef = __shfl(my_coef, min(j, kWave - 1), kWave);
-                if (j < nb) {
+                if (j < n_lead) {
+                    const float2 rc = stage[j];
                     float g[VEC];
-                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)row << kOutShift)) + ch_eff, g);
+                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g);
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coef, g[v], acc[v]);
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(rc.y, g[v], acc[v]);
                 }
             }
+            __builtin_amdgcn_wave_barrier();      // the records are read before the next chunk overwrites them
         }
         // the depth sums sit in the lanes that loaded the pairs: fold them into lane 0
 #pragma unroll
@@ -2449,8 +2472,8 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
     // and room for the depth bin in a pair's first word)
     const int from_pairs =
         (d_depth != nullptr && pl.k.C <= pl.k.lanes_per_slot * pl.vec * pl.cpl && pl.k.bin_bits >= 0) ? 1 : 0;
-    const size_t lds = ((size_t)nw * (lpr * vec + 2) + (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) *
-                       sizeof(float);
+    const size_t lds = ((size_t)texel_waves * kWave * 2 + (size_t)nw * (lpr * vec + 2) +
+                        (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) * sizeof(float);
     long long want_split = kTexelSplitBelow / texels;
     const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);
