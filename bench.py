@@ -47,7 +47,7 @@ HBM_PEAK_GBS = 8000.0
 # counters read for a 256 MiB copy (x2.000 / x1.000); see profiles/.  Only for the workload
 # and kernels the counters were collected on; anything else reports null.
 MEASURED_TRAFFIC = {
-    ("cfg2_surround", "laplace", 0): {"backward": 22.5e6, "forward": 8.40e6,
+    ("cfg2_surround", "laplace", 0): {"backward": 22.4e6, "forward": 8.40e6,
                                       "source": "profiles/cfg2_surround_laplace_fwd_bwd_gather.md"},
 }
 DIST_OF = {"gaussian": (0, "parametric"), "laplace": (1, "parametric"), "categorical": (2, "categorical")}
