@@ -90,6 +90,7 @@ constexpr int kReplicas = 1 << kReplicaBits;
 // With fixed-capacity segments (no counting pass) a texel has four segments, again chosen by cell.
 constexpr int kFixedReplicas = 4;
 constexpr int kFixedMinSegment = 4;           // shorter segments would mostly overflow: count instead
+constexpr long long kStreamOutputFrom = 32ll << 20;   // bytes of forward output beyond what the eight L2s hold
 constexpr int kClaimRunsFrom = 300;           // possible samples per claim counter from which runs claim together
 static_assert(kFixedReplicas == 4, "the texel pass numbers a texel's lists first corner + 4 * replica");
 constexpr int kScanChunkBits = 12;           // counters are prefix-summed in chunks of 4096
@@ -595,7 +596,9 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
 }
 
 // ---------------------------------------------------------------- forward
-template <typename T, int VEC, int CPL>
+// STREAM: the output is stored with non-temporal stores (a template parameter: as a run-time
+// choice between two stores the compiler merges them into one ordinary store).
+template <typename T, int VEC, int CPL, bool STREAM>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     KParams k, const T *__restrict__ depth, const T *__restrict__ feats, const float *__restrict__ proj,
     float *__restrict__ out, float *__restrict__ count_out) {
@@ -724,9 +727,14 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
                             o[ch] = res[0];
                         } else {
 #pragma unroll
-                            for (int v = 0; v < VEC; v += 4)
-                                *reinterpret_cast<float4 *>(o + ch + v) =
-                                    make_float4(res[v], res[v + 1], res[v + 2], res[v + 3]);
+                            for (int v = 0; v < VEC; v += 4) {
+                                // an output too large for the L2s is streamed past them: it is written
+                                // once, and what the next kernel reads stays cached instead
+                                typedef float float4v __attribute__((ext_vector_type(4)));
+                                const float4v row = {res[v], res[v + 1], res[v + 2], res[v + 3]};
+                                if (STREAM) __builtin_nontemporal_store(row, reinterpret_cast<float4v *>(o + ch + v));
+                                else *reinterpret_cast<float4v *>(o + ch + v) = row;
+                            }
                         }
                     }
                 }
@@ -738,9 +746,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
 
 // ---------------------------------------------------------------- backward
 // Two ways to form the feature gradient, which is a sum over all samples that touch a texel:
-//   scatter      fbev_backward_cells_kernel<.., false>: one hardware fp32 atomic per (sample,
+//   scatter      fbev_backward_cells_kernel<.., 0>: one hardware fp32 atomic per (sample,
 //                corner, channel).  Needs no workspace; slow under contention.
-//   inverse map  let the cell pass (fbev_backward_cells_kernel<.., true>) drop one 32-byte record
+//   inverse map  let the cell pass (fbev_backward_cells_kernel<.., 1 or 2>) drop one 32-byte record
 //                per kept sample into the segment of the sample's first corner texel (segments
 //                of fixed capacity, or packed after a counting pass and a prefix sum), then
 //                gather per texel from the segments of the four texels whose samples reach it
@@ -2156,14 +2164,23 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
     prof::Scope timer(out != nullptr ? prof::kForward : prof::kCellCount, st);
-    switch (pl.cpl) {
-        case 1: if (!lds_opt_in(fbev_forward_kernel<T, VEC, 1>, pl.lds_fwd)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 1>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
-        case 2: if (!lds_opt_in(fbev_forward_kernel<T, VEC, 2>, pl.lds_fwd)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 2>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
-        default: if (!lds_opt_in(fbev_forward_kernel<T, VEC, 4>, pl.lds_fwd)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_forward_kernel<T, VEC, 4>), grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt); break;
+    const bool stream = VEC > 1 && (long long)pl.k.B * pl.k.gy * pl.k.gx * pl.k.C * 4 > kStreamOutputFrom;
+    auto launch = [&](auto kernel) {
+        if (!lds_opt_in(kernel, pl.lds_fwd)) return false;
+        hipLaunchKernelGGL(kernel, grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt);
+        return true;
+    };
+    bool ok;
+    if (stream) {
+        constexpr bool S = VEC > 1;      // no streaming instantiations off the vector paths
+        ok = pl.cpl == 1 ? launch(fbev_forward_kernel<T, VEC, 1, S>)
+                         : (pl.cpl == 2 ? launch(fbev_forward_kernel<T, VEC, 2, S>) : launch(fbev_forward_kernel<T, VEC, 4, S>));
+    } else {
+        ok = pl.cpl == 1 ? launch(fbev_forward_kernel<T, VEC, 1, false>)
+                         : (pl.cpl == 2 ? launch(fbev_forward_kernel<T, VEC, 2, false>)
+                                        : launch(fbev_forward_kernel<T, VEC, 4, false>));
     }
+    if (!ok) return FBEV_ERR_LAUNCH;
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
