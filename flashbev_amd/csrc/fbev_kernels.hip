@@ -2069,7 +2069,7 @@ int validate(const fbev_problem *p, bool need_channels) {
     return FBEV_OK;
 }
 
-int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWavesPerBlock, int max_rounds = 8,
+int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWavesPerBlock, int max_rounds = 3,
               int slot_budget = kMaxSlotLdsBytes) {
     const int entry_bytes = 32 + 4;      // an entry (two float4 in every kernel) and its candidate index
     KParams &k = plan->k;
@@ -2117,7 +2117,10 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     k.slots = slots;
     k.groups_per_slot = (kWave / lps) / slots;     // >= 1: slots <= kWave / lps
     k.list_cap = k.NZ;
-    // enough wavefronts to fill 256 CUs several times over before a wavefront takes more rounds
+    // enough wavefronts to fill 256 CUs several times over before a wavefront takes more rounds,
+    // and never many rounds: cells differ widely in their number of samples, and short wavefronts
+    // even that out (training-size cell pass: 439 / 406 / 399 / 404 / 439 us with at most
+    // 8 / 4 / 3 / 2 / 1 rounds; the forward does not care)
     const long long groups = ((long long)k.padded_cells + slots - 1) / slots * k.B;
     int rounds = (int)(groups / (256ll * 4 * 8 * 2));
     k.rounds = rounds < 1 ? 1 : (rounds > max_rounds ? max_rounds : rounds);
