@@ -131,11 +131,16 @@ class SamplingVT(nn.Module):
     @staticmethod
     def _pointwise(conv, x):
         """A 1x1 convolution of ``x [M, C, H, W]`` with channels-last output ``[M, H, W, C_out]``:
-        a matrix product over a transposed view of ``x`` (no copy for either memory format)."""
+        one matrix product over a transposed view of ``x``, bias included, no copy for either memory
+        format (for NCHW input the transposition is left to the batched product's operand flags)."""
         M, C, H, W = x.shape
-        rows = x.permute(0, 2, 3, 1).reshape(M, H * W, C) if x.is_contiguous(memory_format=torch.channels_last) \
-            else x.flatten(2).transpose(1, 2)
-        return F.linear(rows, conv.weight.flatten(1), conv.bias).unflatten(1, (H, W))
+        weight = conv.weight.flatten(1)                                   # [C_out, C]
+        if x.is_contiguous(memory_format=torch.channels_last):
+            return F.linear(x.permute(0, 2, 3, 1).reshape(M, H * W, C), weight, conv.bias).unflatten(1, (H, W))
+        rows = x.flatten(2).transpose(1, 2)                               # [M, H*W, C] view of NCHW
+        w_t = weight.t().expand(M, -1, -1)
+        out = torch.bmm(rows, w_t) if conv.bias is None else torch.baddbmm(conv.bias, rows, w_t)
+        return out.unflatten(1, (H, W))
 
     def _depth_last(self, x):
         d = torch.relu(self._pointwise(self.depth_network[0], x))
