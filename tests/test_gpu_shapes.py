@@ -70,6 +70,18 @@ def test_many_samples_per_cell():
     check_all(w, x, 1, thr=0.0)
 
 
+@pytest.mark.parametrize("dist", [1, 2])
+def test_twelve_cameras_sixteen_cells_per_wavefront(dist):
+    """Four channels leave one lane per cell, so a wavefront takes 16 cells per round; with twelve
+    cameras that is 192 (cell, camera) columns: the column stage of the sample phase runs three
+    times per round, and every second camera overlaps its neighbours."""
+    w = small(yaws=tuple(30.0 * i for i in range(12)), channels=4, grid_size=(24, 24, 2), depth_bins=8)
+    x = make_inputs(w, MODEL[dist], device="cuda", with_grad_out=True)
+    assert x["image_feats"].shape[1] == 12
+    print(f"[case] 12 cameras dist={dist}", flush=True)
+    check_all(w, x, dist, thr=0.0)
+
+
 def test_grid_not_multiple_of_tile_and_unaligned_views():
     w = small(channels=20, grid_size=(37, 19, 5))
     x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
