@@ -1,0 +1,284 @@
+// Backward, texel side of the inverse map.
+// Part of the single translation unit fbev_kernels.hip; not meant to be compiled on its own.
+#pragma once
+
+namespace {
+
+// Texel pass of the inverse-map backward.  The samples that reach texel t are filed under their
+// first corner: t itself, its left neighbour, the texel above, and the one above-left (a sample's
+// corners are (v0|v1, u0|u1) with u1 = u0 + 1 and v1 = v0 + 1 unless clamped).  Those four lists
+// are handled by one block, or, when the grid has a second dimension and a list is longer than
+// kTexelPart, by up to gridDim.y blocks that each take an equal share of every list.  Every block
+// of a texel first has to read the lists' bounds, so idle blocks are not free: the host splits
+// only when there are too few texels to fill the machine otherwise (kTexelSplitBelow).  A block's
+// WAVES * (64 / lanes_per_row) workers stride over the pairs, each gathering grad_out rows with
+// 128-bit loads; partial rows meet in LDS.  A texel handled by one block is updated with plain
+// loads and stores; the shares of a split texel are combined with fp32 atomics (at most
+// gridDim.y per address).
+constexpr int kTexelMaxSplit = 8;
+constexpr int kTexelSplitBelow = 8192;
+constexpr int kTexelPart = 128;
+constexpr int kTexelOneWaveBelow = 100;      // possible samples per texel below which a block is one wavefront ...
+constexpr int kTexelManyTexels = 50000;      // ... or three times that when there are this many texels
+constexpr int kTexelTwoWavesBelow = 450;     // below which it is two wavefronts; four from there on
+constexpr int kTexelSegs = 4 * kFixedReplicas;   // lists of a texel with fixed segments: 4 first corners x replicas
+template <int VEC, int WAVES>
+__global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
+    KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
+    const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
+    float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs, int fresh) {
+    extern __shared__ float4 smem[];
+    // per wavefront 64 (grad_out row, coefficient) records of the chunk in hand, then the partial rows
+    float2 *stage = reinterpret_cast<float2 *>(smem) + (threadIdx.x >> 6) * kWave;
+    float *part = reinterpret_cast<float *>(smem) + WAVES * kWave * 2;
+    // Blocks are dealt to the accelerator dies in turn; let each die walk a contiguous range of
+    // texels, column by column: the texels of a feature-map column gather the cells along one
+    // wedge of rays (a cell's height bins land on neighbouring rows), so their grad_out rows meet
+    // in one L2 while they are still there.
+    // (Measured: 10 % faster at 33 792 texels with 1 KiB rows; at 4224 texels no faster, but the pass
+    // reads 3.7 times less from HBM.)
+    int t = blockIdx.x;
+    if (gridDim.x >= 1024) {
+        const int j = xcd_swizzle(blockIdx.x, gridDim.x), hw = k.H * k.W;
+        const int img = j / hw, rem = j - img * hw, u = rem / k.H, v = rem - u * k.H;
+        t = (img * k.H + v) * k.W + u;
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    constexpr int n_waves = WAVES;
+    const bool counted = chunk_prefix != nullptr;
+    // List e of the texel: first corner (e & 3 with fixed segments, e when counted): bit 0 = one
+    // texel to the left, bit 1 = one row up; replica e >> 2 with fixed segments.  A cell's samples
+    // on neighbouring height bins sit in different lists of the same replica, at about the same
+    // relative position (they were claimed together): replica-major order keeps them close in
+    // time, so the second gather of the cell's grad_out row finds it in cache.
+    // Every wavefront builds the table for itself in its first kTexelSegs lanes (lane e holds list
+    // e): no LDS, no barrier before the first pair is requested.
+    const int tu = t % k.W, tv = (t / k.W) % k.H;
+    int my_lo = 0, my_len = 0;
+    bool spilled = false;      // a list of this texel was full: the cell pass added the rest with atomics
+    if (lane < kTexelSegs) {
+        const int e = lane;
+        const int o = counted ? e : e & 3;
+        const bool exists = (counted ? e < 4 : true) && (!(o & 1) || tu > 0) && (!(o & 2) || tv > 0);
+        const int q = t - (o & 1) - ((o & 2) ? k.W : 0);
+        if (exists && counted) {
+            // counted segments, one after the other: from the end of the previous texel's last
+            // replica to the end of this texel's
+            const long long first = (long long)q * kReplicas - 1, last = (long long)q * kReplicas + kReplicas - 1;
+            my_lo = q == 0 ? 0 : chunk_prefix[first >> kScanChunkBits] + seg_end[first];
+            const int list_end = chunk_prefix[last >> kScanChunkBits] + seg_end[last];
+            spilled = list_end > pair_cap;
+            my_len = max(min(list_end, pair_cap) - my_lo, 0);
+        } else if (exists) {
+            // fixed segments of pair_cap pairs; seg_end holds how many were claimed
+            const int i = q * kFixedReplicas + (e >> 2);
+            my_lo = i * pair_cap;
+            const int claimed = seg_end[i];
+            spilled = claimed > pair_cap;
+            my_len = max(min(claimed, pair_cap), 0);
+        }
+    }
+    // the lists one after the other form one sequence of pairs; list e starts at my_pre of lane e
+    int my_pre = my_len;
+#pragma unroll
+    for (int off = 1; off < kTexelSegs; off <<= 1) {
+        const int other = __shfl_up(my_pre, off, kWave);
+        if (lane >= off) my_pre += other;
+    }
+    my_pre -= my_len;                              // exclusive
+    int list_start[kTexelSegs];                    // wave-uniform copies of the starts of lists 1 ..
+#pragma unroll
+    for (int j = 1; j < kTexelSegs; ++j) list_start[j] = __builtin_amdgcn_readlane(my_pre, j);
+    const int n_all = __builtin_amdgcn_readlane(my_pre, kTexelSegs - 1) + __builtin_amdgcn_readlane(my_len, kTexelSegs - 1);
+    const int n_parts = min((int)gridDim.y, (n_all + 4 * kTexelPart - 1) / (4 * kTexelPart));
+    if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
+    const bool shared_texel = n_parts > 1;
+    // The gradient buffers were cleared by this call (fresh) and nothing but this block touches the
+    // texel unless a list spilled: then its rows are stored, not added, and the pass ends without a
+    // dependent load.
+    const bool store_only = fresh != 0 && !shared_texel && __ballot(spilled) == 0ull;
+    const int part_lo = (int)(((long long)n_all * blockIdx.y) / n_parts);
+    const int part_hi = (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
+    // the wavefronts take chunks of the sequence in turn: 64 pairs, fewer when that leaves a wavefront idle
+    const int chunk = min(kWave, max(1, (part_hi - part_lo + n_waves - 1) / n_waves));
+    const unsigned n_cells = (unsigned)(k.B * k.gy * k.gx);
+    const int wpw = kWave / lanes_per_row;            // workers per wavefront
+    const int nw = wpw * n_waves;
+    const int wslot = lane / lanes_per_row;
+    const int lir = lane - wslot * lanes_per_row;
+    const bool worker_lane = wslot < wpw;
+    const int worker = wave * wpw + wslot;
+    const int span = lanes_per_row * VEC;
+    const int stride = span + 2;                      // partial row + the two depth sums
+    // categorical depth gradient: one LDS accumulator per depth bin of this texel
+    const bool bin_sums = depth_from_pairs && k.dist == FBEV_CATEGORICAL;
+    float *bins = part + nw * stride;
+    const int bin_bits = depth_from_pairs ? k.bin_bits : 0, bin_mask = (1 << bin_bits) - 1;
+    if (bin_sums) {
+        for (int i = threadIdx.x; i < k.Dd; i += blockDim.x) bins[i] = 0.0f;
+        __syncthreads();
+    }
+    constexpr int kOutShift = VEC > 1 ? 4 : 2;
+    const unsigned out_units = (unsigned)(VEC > 1 ? k.C / 4 : k.C);
+    const char *gbytes = reinterpret_cast<const char *>(grad_out);
+    for (int c0 = 0; c0 < k.C; c0 += span) {
+        const int ch = c0 + lir * VEC;
+        const bool on = worker_lane && ch < k.C;
+        const int ch_eff = on ? ch : 0, wslot_eff = min(wslot, wpw - 1);
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+        float sa = 0.0f, sb = 0.0f;
+        // A wavefront takes 64 consecutive pairs at a time, one per lane in a single coalesced
+        // load, and hands them to its workers through 512 bytes of LDS; four grad_out rows per
+        // worker are in flight before the first is used.  The loop is bound by load latency:
+        // without this the pair load and the row load it addresses form a dependent chain.
+        for (int bstart = part_lo + wave * chunk; bstart < part_hi; bstart += n_waves * chunk) {
+            const int nb = min(chunk, part_hi - bstart);
+            float4 pr = make_float4(__int_as_float(-1), 0.f, 0.f, 0.f), pd = make_float4(0.f, 0.f, 0.f, 0.f);
+            // which list position bstart + lane falls into (all lanes take part in the shuffles;
+            // positions past the chunk fall into some list and are not loaded)
+            const int vi = bstart + lane;
+            int e = 0;
+#pragma unroll
+            for (int j = 1; j < kTexelSegs; ++j) e += vi >= list_start[j] ? 1 : 0;
+            const int o = counted ? e : e & 3;
+            // lane e of the wavefront knows where list e lies in the pair array
+            const int src_pos = __shfl(my_lo, e, kWave) + (vi - __shfl(my_pre, e, kWave));
+            if (lane < nb) {
+                const float4 *src = reinterpret_cast<const float4 *>(pairs + src_pos);
+                pr = src[0];
+                pd = src[1];
+            }
+            const int word = __float_as_int(pr.x);
+            // a pair is written by the cell pass before this kernel starts; the range check only
+            // keeps a logic error from turning into a wild read (such a pair counts as cell 0
+            // with coefficient 0)
+            const bool valid = (unsigned)(word >> bin_bits) < n_cells;
+            // the sample's bilinear weight on this texel: the corners that land here (a clamped
+            // corner stays on the first corner's column / row)
+            const float du = pr.z, dv = pr.w;
+            const bool fu = __float_as_int(pd.z) & 1, fv = __float_as_int(pd.z) & 2;
+            const float w00 = (1.0f - du) * (1.0f - dv), w01 = (1.0f - du) * dv, w10 = du * (1.0f - dv), w11 = du * dv;
+            float cw;
+            if (o == 0) cw = w00 + (fu ? 0.0f : w10) + (fv ? 0.0f : w01) + ((fu || fv) ? 0.0f : w11);
+            else if (o == 1) cw = fu ? w10 + (fv ? 0.0f : w11) : 0.0f;
+            else if (o == 2) cw = fv ? w01 + (fu ? 0.0f : w11) : 0.0f;
+            else cw = (fu && fv) ? w11 : 0.0f;
+            // where the pair's grad_out row starts, in units of 16 bytes (one float off the vector path)
+            const unsigned my_row = valid ? (unsigned)(word >> bin_bits) * out_units : 0u;
+            const float my_coef = valid ? pr.y * cw : 0.0f;
+            if (c0 == 0 && valid) {
+                if (bin_sums) {
+                    const int k0 = word & bin_mask;
+                    __hip_atomic_fetch_add(bins + k0, pd.x * cw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(bins + min(k0 + 1, k.Dd - 1), pd.y * cw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                } else {
+                    sa += pd.x * cw;
+                    sb += pd.y * cw;
+                }
+            }
+            // Pairs that follow each other in a list and come from one cell (its samples on
+            // neighbouring height bins that share a first corner claimed neighbouring positions)
+            // gather the same grad_out row: their coefficients are added up and the row is
+            // gathered once.  A run gets a new leader every eight lanes, so that three steps of a
+            // suffix sum inside the runs leave every leader with its run's coefficient.
+            const unsigned prev_row = (unsigned)__shfl_up((int)my_row, 1, kWave);
+            const bool in_chunk = lane < nb;
+            const unsigned long long cm = __ballot(in_chunk && lane > 0 && my_row == prev_row);
+            const int run_lead = 63 - __clzll(~cm & lanemask_le(lane));
+            const unsigned long long lm = __ballot(in_chunk && ((lane - run_lead) & 7) == 0);
+            const unsigned long long later = lane == 63 ? 0ull : (lm >> (lane + 1));      // leaders after me
+            const int followers = later ? __ffsll((long long)later) - 1 : 63 - lane;    // lanes past the chunk carry 0
+            float run_coef = my_coef;
+#pragma unroll
+            for (int off = 1; off <= 4; off <<= 1) {
+                const float other = __shfl_down(run_coef, off, kWave);
+                if (off <= followers) run_coef += other;
+            }
+            const int n_lead = __popcll(lm);
+            if ((lm >> lane) & 1ull) stage[__popcll(lm & lanemask_lt(lane))] = make_float2(__int_as_float((int)my_row), run_coef);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            // Full groups of UNR rows per worker run without predicates (lanes that carry no
+            // channel gather channel 0 of some row and drop the result); the remainder goes one
+            // row per worker.
+            constexpr int UNR = 4;
+            const int group = wpw * UNR, full = n_lead - n_lead % group;
+            for (int i = 0; i < full; i += group) {
+                float coefs[UNR];
+                float g[UNR][VEC];
+#pragma unroll
+                for (int q = 0; q < UNR; ++q) {
+                    const float2 rc = stage[i + q * wpw + wslot_eff];
+                    coefs[q] = rc.y;
+                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g[q]);
+                }
+#pragma unroll
+                for (int q = 0; q < UNR; ++q)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coefs[q], g[q][v], acc[v]);
+            }
+            for (int i = full; i < n_lead; i += wpw) {
+                const int j = i + wslot_eff;
+                if (j < n_lead) {
+                    const float2 rc = stage[j];
+                    float g[VEC];
+                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g);
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(rc.y, g[v], acc[v]);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();      // the records are read before the next chunk overwrites them
+        }
+        // the depth sums sit in the lanes that loaded the pairs: fold them into lane 0
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            sa += __shfl_xor(sa, off, kWave);
+            sb += __shfl_xor(sb, off, kWave);
+        }
+        __syncthreads();   // previous pass has been read
+        if (worker_lane) {
+            if (ch < k.C) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) part[worker * stride + lir * VEC + v] = acc[v];
+            }
+            if (lir == 0) {
+                part[worker * stride + span] = wslot == 0 ? sa : 0.0f;
+                part[worker * stride + span + 1] = wslot == 0 ? sb : 0.0f;
+            }
+        }
+        __syncthreads();
+        for (int c = threadIdx.x; c < span && c0 + c < k.C; c += blockDim.x) {
+            float sum = 0.0f;
+            for (int w = 0; w < nw; ++w) sum += part[w * stride + c];
+            if (d_feats != nullptr) {
+                float *dst = d_feats + (size_t)t * k.C + c0 + c;
+                if (shared_texel) atomic_add_f32(dst, sum);
+                else if (store_only) *dst = sum;
+                else *dst += sum;
+            }
+        }
+        if (c0 == 0 && bin_sums) {
+            for (int i = threadIdx.x; i < k.Dd; i += blockDim.x) {
+                const float sum = bins[i];
+                if (sum != 0.0f) {
+                    float *dst = d_depth + (size_t)t * k.Dd + i;
+                    if (shared_texel) atomic_add_f32(dst, sum);
+                    else if (store_only) *dst = sum;
+                    else *dst += sum;
+                }
+            }
+        } else if (c0 == 0 && depth_from_pairs && threadIdx.x < 2) {
+            float sum = 0.0f;
+            for (int w = 0; w < nw; ++w) sum += part[w * stride + span + threadIdx.x];
+            float *dst = d_depth + (size_t)t * 2 + threadIdx.x;
+            if (shared_texel) atomic_add_f32(dst, sum);
+            else if (store_only) *dst = sum;
+            else *dst += sum;
+        }
+    }
+}
+
+}  // namespace

@@ -1,0 +1,292 @@
+// The sample phase of the cell-centric kernels (forward, backward cell pass, count): a
+// wavefront's LDS view and the three-stage evaluation of the samples of its cells.
+// Part of the single translation unit fbev_kernels.hip; not meant to be compiled on its own.
+#pragma once
+
+namespace {
+
+// LDS of one block of the cell-centric kernels (float4 units):
+//   [matrices: N*12 floats][column table: slots*N ints]
+//   per wavefront: [16 ints of list lengths][16 float4 of cell centres][slots*N column records]
+//   [slots*N ints: columns in view][slots*NZ ints of candidates][slots * list_cap entries]
+// Counters that several lanes of a wavefront update in turn live in LDS and are read as
+// volatile.  The pointer carries the LDS address space: a volatile access through a generic
+// pointer becomes a system-coherent flat load that first waits for every outstanding global
+// store and atomic of the wavefront.
+using lds_counter = volatile __attribute__((address_space(3))) int;
+
+struct WaveLds {
+    const float *Pm;
+    const int *dec;       // column index within the wavefront's round -> slot << 28 | camera << 16
+    lds_counter *cnt;     // entries per slot
+    float4 *cell;         // per slot: x, y, valid flag, ix | iy << 16
+    float4 *col;          // per column: the (x, y) part of U, V, D, and its dec word
+    int *alive;           // columns with a height bin that may be in view
+    unsigned *cand;       // samples that survive the cheap test: column << 16 | height bin
+    float4 *lst;
+};
+
+__device__ __forceinline__ int lds_p_f4(const KParams &k) { return (k.N * 12 + 3) / 4; }
+__device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots * k.N + 3) / 4; }
+__device__ __forceinline__ int lds_cand_f4(const KParams &k) { return (k.slots * k.NZ + 3) / 4; }
+
+// Stage the block's matrices and the column table; returns the wavefront's view.  Ends with a
+// barrier.
+__device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *smem, const float *__restrict__ proj,
+                                                   int b, int entry_f4) {
+    WaveLds L;
+    float *Pm = reinterpret_cast<float *>(smem);
+    int *dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
+    const int dec_f4 = lds_dec_f4(k), cand_f4 = lds_cand_f4(k), cols = k.slots * k.N;
+    const int per_wave_f4 = 4 + 16 + cols + dec_f4 + cand_f4 + k.slots * k.list_cap * entry_f4;
+    float4 *wbase = smem + lds_p_f4(k) + dec_f4 + (threadIdx.x >> 6) * per_wave_f4;
+    L.Pm = Pm;
+    L.dec = dec;
+    L.cnt = (lds_counter *)reinterpret_cast<int *>(wbase);
+    L.cell = wbase + 4;
+    L.col = wbase + 20;
+    L.alive = reinterpret_cast<int *>(wbase + 20 + cols);
+    L.cand = reinterpret_cast<unsigned *>(wbase + 20 + cols + dec_f4);
+    L.lst = wbase + 20 + cols + dec_f4 + cand_f4;
+    for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
+        Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        const int slot = i / k.N, cam = i - slot * k.N;
+        dec[i] = (slot << 28) | (cam << 16);
+    }
+    __syncthreads();
+    return L;
+}
+
+// Entry of a compacted list: ENTRY_F4 float4 words.
+//   forward   word 0: corner weights already multiplied by the depth weight
+//             word 1: where the four texels' feature rows start, in address units (texel index
+//                     ((b*N+n)*H + v)*W + u times KParams::row_units) as int bits (t00, t01, t10, t11):
+//                     the gather loop then forms an address with one shift-add, not a 64-bit multiply
+//   backward  word 0: du, dv, t00, (u1 != u0) | (v1 != v0) << 1 -- the four weights and texels
+//                     follow from these exactly as phase A computed them.  Inverse map: t00 << 2 with
+//                     the two flags below it, and in the fourth place the position of the sample's
+//                     pair in the pair array (sorted by first corner texel), or -1 if the array is full
+//             word 1: wgt, a, b, (k0 | k1 << 16)
+enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeFillRuns = 4 };
+
+// Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
+// pixel coordinate misses the image by more than this fraction, far beyond any rounding of
+// the exact test it would otherwise take (and fail).
+constexpr float kEarlySlack = 1.0e-3f;
+
+// Phase A of one round of a wavefront: the samples of its `slots` cells, in three stages.
+//   stage 0  lanes = (cell, camera) columns: the (x, y) part of the three dot products, shared by
+//            the column's height bins, and a test of the column's two end bins.  U, V and D are
+//            monotone in the height bin (every rounded operation is), so a column whose end bins
+//            both miss the image on the same side, or both lie behind the camera, holds no sample
+//            that stage 1 could pass.  About three columns in four end here.
+//   stage 1  lanes = height bins of the remaining columns: the rest of the dot products and a
+//            division-free test that can only reject samples the exact test rejects too (behind
+//            the camera, or outside the image by more than kEarlySlack).  Survivors are compacted,
+//            in order, into the candidate list.
+//   stage 2  lanes = candidates, densely packed: the canonical arithmetic (divisions, floor,
+//            bilinear weights), the depth model, the weight threshold; what is kept goes, still
+//            in (camera, height) order, into its slot's entry list.
+// kModeCount writes no entries; it only counts the kept samples per (first-corner texel, replica).
+template <int ENTRY_F4, typename T, int MODE>
+__device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, const T *__restrict__ depth, int b, int q0,
+                                        int lane, const int *__restrict__ chunk_prefix = nullptr,
+                                        int *__restrict__ cursor = nullptr, int pair_cap = 0) {
+    constexpr bool FILLING = MODE == kModeFill || MODE == kModeFillRuns;   // the latter claims per run
+    constexpr bool BACKWARD = MODE == kModeScatter || FILLING;
+    const int n_cols = k.slots * k.N;
+    if (lane < 16) L.cnt[lane] = 0;
+    if (lane < k.slots) {
+        int ix = 0, iy = 0;
+        const bool ok = cell_of(k, q0 + lane, ix, iy);
+        L.cell[lane] = make_float4(voxel_coord(k.xmin, ix, k.vx), voxel_coord(k.ymin, iy, k.vy), ok ? 1.0f : 0.0f,
+                                   __int_as_float(ix | (iy << 16)));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    const float u_max = k.Wi_f * (1.0f + kEarlySlack), v_max = k.Hi_f * (1.0f + kEarlySlack);
+    // ---- stage 0
+    int n_alive = 0;
+    const float z_first = voxel_coord(k.zmin, 0, k.vz), z_last = voxel_coord(k.zmin, k.gz - 1, k.vz);
+    for (int base = 0; base < n_cols; base += kWave) {
+        const int cc = base + lane;
+        bool alive = false;
+        if (cc < n_cols) {
+            const int code = L.dec[cc];
+            const float4 c = L.cell[(code >> 28) & 15];
+            if (c.z != 0.0f) {
+                const float *P = L.Pm + ((code >> 16) & 0xfff) * 12;
+                const float au = P[0] * c.x + P[1] * c.y, av = P[4] * c.x + P[5] * c.y, ad = P[8] * c.x + P[9] * c.y;
+                L.col[cc] = make_float4(au, av, ad, __int_as_float(code));
+                const float d0 = (ad + P[10] * z_first) + P[11], d1 = (ad + P[10] * z_last) + P[11];
+                const float d_hi = fmaxf(d0, d1);
+                if (d_hi > 0.0f) {
+                    const float u0 = (au + P[2] * z_first) + P[3], u1 = (au + P[2] * z_last) + P[3];
+                    const float v0 = (av + P[6] * z_first) + P[7], v1 = (av + P[6] * z_last) + P[7];
+                    // stage 1 compares every bin with bounds that grow with its clamped depth
+                    const float dc = fmaxf(d_hi, k.eps), lo = -kEarlySlack * dc;
+                    alive = fmaxf(u0, u1) >= lo && fminf(u0, u1) <= u_max * dc && fmaxf(v0, v1) >= lo &&
+                            fminf(v0, v1) <= v_max * dc;
+                }
+            }
+        }
+        const unsigned long long m = __ballot(alive);
+        if (alive) L.alive[n_alive + __popcll(m & lanemask_lt(lane))] = cc;
+        n_alive += __popcll(m);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- stage 1
+    int n_cand = 0;
+    const int total = n_alive * k.gz;
+    for (int base = 0; base < total; base += kWave) {
+        const int idx = base + lane;
+        bool pass = false;
+        unsigned key = 0;
+        if (idx < total) {
+            const int a = (int)(__umul24((unsigned)idx, (unsigned)k.gz_magic) >> k.gz_shift);
+            const int iz = idx - a * k.gz;
+            const int cc = L.alive[a];
+            const float4 col = L.col[cc];
+            const float *P = L.Pm + ((__float_as_int(col.w) >> 16) & 0xfff) * 12;
+            const float z = voxel_coord(k.zmin, iz, k.vz);
+            const float D = (col.z + P[10] * z) + P[11];
+            key = ((unsigned)cc << 16) | (unsigned)iz;
+            if (D > 0.0f) {
+                const float U = (col.x + P[2] * z) + P[3];
+                const float V = (col.y + P[6] * z) + P[7];
+                const float dc = fmaxf(D, k.eps), lo = -kEarlySlack * dc;
+                pass = U >= lo && U <= u_max * dc && V >= lo && V <= v_max * dc;
+            }
+        }
+        const unsigned long long m = __ballot(pass);
+        if (pass) L.cand[n_cand + __popcll(m & lanemask_lt(lane))] = key;
+        n_cand += __popcll(m);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- stage 2
+    for (int base = 0; base < n_cand; base += kWave) {
+        const int j = base + lane;
+        const bool active = j < n_cand;
+        const unsigned key = active ? L.cand[j] : 0u;
+        const float4 col = active ? L.col[key >> 16] : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int d = __float_as_int(col.w);
+        const int slot = active ? (d >> 28) & 15 : 16 + (lane & 1);   // idle lanes: no real slot
+        const int cam = (d >> 16) & 0xfff;
+        float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w2 = w0;
+        int4 tx = make_int4(0, 0, 0, 0);
+        int cellxy = 0;
+        bool keep = false;
+        if (active) {
+            const float4 c = L.cell[slot];
+            cellxy = __float_as_int(c.w);
+            Geom g = project_column(k, L.Pm + cam * 12, col.x, col.y, col.z, voxel_coord(k.zmin, key & 0xffffu, k.vz));
+            if (g.valid) {
+                float w00 = (1.0f - g.du) * (1.0f - g.dv);
+                float w01 = (1.0f - g.du) * g.dv;
+                float w10 = g.du * (1.0f - g.dv);
+                float w11 = g.du * g.dv;
+                int rowbase = (b * k.N + cam) * k.H;
+                int t00 = (rowbase + g.v0) * k.W + g.u0;
+                int t01 = (rowbase + g.v1) * k.W + g.u0;
+                int t10 = (rowbase + g.v0) * k.W + g.u1;
+                int t11 = (rowbase + g.v1) * k.W + g.u1;
+                DepthEval e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
+                keep = e.keep;
+                tx = make_int4(t00, t01, t10, t11);
+                if (BACKWARD) {
+                    const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
+                    w0 = FILLING ? make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1))
+                                           : make_float4(g.du, g.dv, __int_as_float(t00), __int_as_float(fl));
+                    w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
+                } else {
+                    w0 = make_float4(w00 * e.wgt, w01 * e.wgt, w10 * e.wgt, w11 * e.wgt);
+                }
+            }
+        }
+        const int prev_slot = __shfl_up(slot, 1, kWave);
+        // Consecutive height bins of one (cell, camera) often fall on the same texel (far cells
+        // compress onto the horizon rows).  Samples that repeat the first corner of the previous
+        // kept sample of the same cell form a run; when counting, the run's first lane adds the
+        // whole run with ONE atomic.  Positions are claimed per run as well where a claim counter
+        // may get hundreds of samples (kModeFillRuns): claims on one address are served one
+        // after the other, and a 400 x 400 x 12 grid on 4224 texels spent half of the cell pass
+        // waiting for them.  Elsewhere the shuffles cost more than the saved returning atomics.
+        int run_lead = lane, run_len = 1;
+        if (MODE == kModeCount || MODE == kModeFillRuns) {
+            const int prev_keep = __shfl_up((int)keep, 1, kWave);
+            const int prev_texel = __shfl_up(tx.x, 1, kWave);      // every lane takes part in the exchange
+            const bool cont = keep && lane > 0 && prev_keep != 0 && prev_slot == slot && prev_texel == tx.x;
+            const unsigned long long cm = __ballot(cont);
+            // first lane of my run: the highest lane at or below me that does not continue
+            run_lead = 63 - __clzll(~cm & lanemask_le(lane));
+            // lanes after me that continue without a gap
+            const unsigned long long after = lane == 63 ? 0ull : (cm >> (lane + 1));
+            run_len = 1 + (~after == 0ull ? 63 - lane : __ffsll((long long)~after) - 1);
+        }
+        if (MODE == kModeCount) {
+            if (keep && run_lead == lane)
+                atomicAdd(cursor + tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16), run_len);
+            continue;
+        }
+        // candidates are in sample order, so the lanes of one slot are contiguous: [lo, hi)
+        const unsigned long long bm = __ballot(lane == 0 || slot != prev_slot);
+        const unsigned long long m = __ballot(keep);
+        const int lo = 63 - __clzll(bm & lanemask_le(lane));
+        const unsigned long long above = lane == 63 ? 0ull : (bm & ~lanemask_le(lane));
+        const int hi = above ? __ffsll((long long)above) - 1 : kWave;
+        const unsigned long long seg = (~0ull << lo) & (hi >= 64 ? ~0ull : ((1ull << hi) - 1ull));
+        const int prefix = __popcll(m & seg & lanemask_lt(lane));
+        const int old = active ? L.cnt[slot] : 0;
+        if (keep) {
+            float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
+            e[0] = w0;
+            e[1] = BACKWARD ? w2
+                            : make_float4(__int_as_float(tx.x * k.row_units), __int_as_float(tx.y * k.row_units),
+                                          __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
+        }
+        if (MODE == kModeFill && keep) {
+            // claim the sample's position in the list of its first corner texel
+            int pos;
+            if (chunk_prefix != nullptr) {
+                // counted segments: cursor holds each segment's start within its scan chunk
+                const int i0 = tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16);
+                pos = atomicAdd(cursor + i0, 1) + chunk_prefix[i0 >> kScanChunkBits];
+                pos = pos < pair_cap ? pos : -1;
+            } else {
+                // fixed segments of pair_cap pairs per (texel, replica): cursor counts from zero
+                const int i0 = tx.x * kFixedReplicas + (replica_of(cellxy & 0xffff, cellxy >> 16) & (kFixedReplicas - 1));
+                pos = atomicAdd(cursor + i0, 1);
+                pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
+            }
+            reinterpret_cast<int *>(L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4)[3] = pos;
+        }
+        if (MODE == kModeFillRuns) {
+            // the same, but the run's first lane claims for the whole run (same cell and texel: same
+            // counter) and hands the positions out; every lane takes part in the exchange
+            const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
+            const bool counted = chunk_prefix != nullptr;
+            const int i0 = counted ? tx.x * kReplicas + rep : tx.x * kFixedReplicas + (rep & (kFixedReplicas - 1));
+            int pos = 0;
+            if (keep && run_lead == lane) pos = atomicAdd(cursor + i0, run_len);
+            pos = __shfl(pos, run_lead, kWave) + (lane - run_lead);
+            if (keep) {
+                if (counted) {
+                    pos += chunk_prefix[i0 >> kScanChunkBits];
+                    pos = pos < pair_cap ? pos : -1;
+                } else {
+                    pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
+                }
+                reinterpret_cast<int *>(L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4)[3] = pos;
+            }
+        }
+        if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
+    }
+}
+
+}  // namespace
