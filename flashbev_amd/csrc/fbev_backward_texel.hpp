@@ -16,7 +16,7 @@ namespace {
 // loads and stores; the shares of a split texel are combined with fp32 atomics (at most
 // gridDim.y per address).
 constexpr int kTexelMaxSplit = 8;
-constexpr int kTexelSplitBelow = 8192;
+constexpr int kTexelSplitBelow = 16384;     // texels * blocks per texel stay below this (400x400x12 grid on 4224 texels: 1 / 3 / 7 blocks per texel 107 / 101 / 127 us)
 constexpr int kTexelPart = 128;
 constexpr int kTexelOneWaveBelow = 100;      // possible samples per texel below which a block is one wavefront ...
 constexpr int kTexelManyTexels = 50000;      // ... or three times that when there are this many texels
