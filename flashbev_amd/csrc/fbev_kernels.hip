@@ -343,7 +343,7 @@ int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, co
     // measured: the forward is fastest with at most 4 rounds per wavefront, the backward's cell pass with 8
     // More cells per round pay for the LDS here (measured with 64 channels on a 400x400 grid: 20 height bins
     // 185 -> 166 us, 40 bins 785 -> 476 us); the cell pass of the backward is better off with the smaller budget.
-    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kWavesPerBlock, 4);
+    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kCellPassWaves, 4);
     if (rc != FBEV_OK) return rc;
     return dispatch_forward(p, pl, depth, feats, proj, out, count_out, static_cast<hipStream_t>(stream));
 }
