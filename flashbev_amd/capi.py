@@ -28,7 +28,7 @@ class FbevProblem(ctypes.Structure):
         ("feat_h", ctypes.c_int32), ("feat_w", ctypes.c_int32), ("channels", ctypes.c_int32),
         ("image_h", ctypes.c_int32), ("image_w", ctypes.c_int32),
         ("grid_x", ctypes.c_int32), ("grid_y", ctypes.c_int32), ("grid_z", ctypes.c_int32),
-        ("voxel_min", ctypes.c_float * 3), ("voxel_size", ctypes.c_float * 3),
+        ("voxel_min", ctypes.c_double * 3), ("voxel_size", ctypes.c_double * 3),
         ("epsilon", ctypes.c_float), ("depth_weight_threshold", ctypes.c_float),
         ("depth_distribution", ctypes.c_int32), ("depth_bins", ctypes.c_int32),
         ("depth_min", ctypes.c_float), ("depth_step", ctypes.c_float),

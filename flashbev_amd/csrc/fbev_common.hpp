@@ -85,7 +85,7 @@ struct KParams {
     int groups_per_slot; // lane groups that share a slot's list (more than one when long lists leave few slots)
     int list_cap;        // entries per slot list (= NZ)
     float Wi_f, Hi_f, W_f, H_f;
-    float xmin, ymin, zmin, vx, vy, vz;
+    double xmin, ymin, zmin, vx, vy, vz;   // region of interest and cell size in float64 (see voxel_coord)
     float eps, thr;
     int dist, Dd;
     float dmin, dstep;
@@ -192,8 +192,13 @@ __device__ __forceinline__ Geom project_sample(const KParams &k, const float *P,
     return project_column(k, P, P[0] * x + P[1] * y, P[4] * x + P[5] * y, P[8] * x + P[9] * y, z);
 }
 
-__device__ __forceinline__ float voxel_coord(float lo, int i, float step) {
-    return lo + ((float)i + 0.5f) * step;
+// Centre of cell i along one axis: evaluated in float64 and rounded once to fp32, so that it is the
+// correctly rounded value of lo + (i + 0.5) * (hi - lo) / n.  An fp32 step would carry its rounding
+// error i times along the axis (0.8 m is not an fp32 number), and a Gaussian tail weight multiplies
+// that by z^2.  One float64 multiply-add per cell (x, y) and per height bin of a block (z, kept in
+// an LDS table); nothing per sample.
+__device__ __forceinline__ float voxel_coord(double lo, int i, double step) {
+    return (float)(lo + ((double)i + 0.5) * step);
 }
 
 __device__ __forceinline__ float bilerp(float w00, float w01, float w10, float w11,

@@ -157,9 +157,9 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     k.n_blocks = k.blocks_per_batch * k.B;
     const size_t p_f4 = (size_t)(k.N * 12 + 3) / 4;
     const size_t cols = (size_t)k.slots * k.N, dec_f4 = (cols + 3) / 4;
-    const size_t cand_f4 = ((size_t)k.slots * k.NZ + 3) / 4;
+    const size_t cand_f4 = ((size_t)k.slots * k.NZ + 3) / 4, z_f4 = ((size_t)k.gz + 3) / 4;
     auto block_lds = [&](int entry_f4) {
-        return (p_f4 + dec_f4 +
+        return (p_f4 + dec_f4 + z_f4 +
                 (size_t)waves * (20 + cols + dec_f4 + cand_f4 + (size_t)k.slots * k.list_cap * entry_f4)) * 16;
     };
     {

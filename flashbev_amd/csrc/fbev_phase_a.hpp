@@ -6,7 +6,7 @@
 namespace {
 
 // LDS of one block of the cell-centric kernels (float4 units):
-//   [matrices: N*12 floats][column table: slots*N ints]
+//   [matrices: N*12 floats][column table: slots*N ints][height table: gz floats]
 //   per wavefront: [16 ints of list lengths][16 float4 of cell centres][slots*N column records]
 //   [slots*N ints: columns in view][slots*NZ ints of candidates][slots * list_cap entries]
 // Counters that several lanes of a wavefront update in turn live in LDS and are read as
@@ -18,6 +18,7 @@ using lds_counter = volatile __attribute__((address_space(3))) int;
 struct WaveLds {
     const float *Pm;
     const int *dec;       // column index within the wavefront's round -> slot << 28 | camera << 16
+    const float *zt;      // height bin -> z of the bin's centre
     lds_counter *cnt;     // entries per slot
     float4 *cell;         // per slot: x, y, valid flag, ix | iy << 16
     float4 *col;          // per column: the (x, y) part of U, V, D, and its dec word
@@ -29,8 +30,9 @@ struct WaveLds {
 __device__ __forceinline__ int lds_p_f4(const KParams &k) { return (k.N * 12 + 3) / 4; }
 __device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots * k.N + 3) / 4; }
 __device__ __forceinline__ int lds_cand_f4(const KParams &k) { return (k.slots * k.NZ + 3) / 4; }
+__device__ __forceinline__ int lds_z_f4(const KParams &k) { return (k.gz + 3) / 4; }
 
-// Stage the block's matrices and the column table; returns the wavefront's view.  Ends with a
+// Stage the block's matrices, the column table and the height table; returns the wavefront's view.  Ends with a
 // barrier.
 __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *smem, const float *__restrict__ proj,
                                                    int b, int entry_f4) {
@@ -39,9 +41,11 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
     int *dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
     const int dec_f4 = lds_dec_f4(k), cand_f4 = lds_cand_f4(k), cols = k.slots * k.N;
     const int per_wave_f4 = 4 + 16 + cols + dec_f4 + cand_f4 + k.slots * k.list_cap * entry_f4;
-    float4 *wbase = smem + lds_p_f4(k) + dec_f4 + (threadIdx.x >> 6) * per_wave_f4;
+    float *zt = reinterpret_cast<float *>(smem + lds_p_f4(k) + dec_f4);
+    float4 *wbase = smem + lds_p_f4(k) + dec_f4 + lds_z_f4(k) + (threadIdx.x >> 6) * per_wave_f4;
     L.Pm = Pm;
     L.dec = dec;
+    L.zt = zt;
     L.cnt = (lds_counter *)reinterpret_cast<int *>(wbase);
     L.cell = wbase + 4;
     L.col = wbase + 20;
@@ -54,6 +58,7 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
         const int slot = i / k.N, cam = i - slot * k.N;
         dec[i] = (slot << 28) | (cam << 16);
     }
+    for (int i = threadIdx.x; i < k.gz; i += blockDim.x) zt[i] = voxel_coord(k.zmin, i, k.vz);
     __syncthreads();
     return L;
 }
@@ -109,7 +114,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
     const float u_max = k.Wi_f * (1.0f + kEarlySlack), v_max = k.Hi_f * (1.0f + kEarlySlack);
     // ---- stage 0
     int n_alive = 0;
-    const float z_first = voxel_coord(k.zmin, 0, k.vz), z_last = voxel_coord(k.zmin, k.gz - 1, k.vz);
+    const float z_first = L.zt[0], z_last = L.zt[k.gz - 1];
     for (int base = 0; base < n_cols; base += kWave) {
         const int cc = base + lane;
         bool alive = false;
@@ -152,7 +157,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
             const int cc = L.alive[a];
             const float4 col = L.col[cc];
             const float *P = L.Pm + ((__float_as_int(col.w) >> 16) & 0xfff) * 12;
-            const float z = voxel_coord(k.zmin, iz, k.vz);
+            const float z = L.zt[iz];
             const float D = (col.z + P[10] * z) + P[11];
             key = ((unsigned)cc << 16) | (unsigned)iz;
             if (D > 0.0f) {
@@ -185,7 +190,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         if (active) {
             const float4 c = L.cell[slot];
             cellxy = __float_as_int(c.w);
-            Geom g = project_column(k, L.Pm + cam * 12, col.x, col.y, col.z, voxel_coord(k.zmin, key & 0xffffu, k.vz));
+            Geom g = project_column(k, L.Pm + cam * 12, col.x, col.y, col.z, L.zt[key & 0xffffu]);
             if (g.valid) {
                 float w00 = (1.0f - g.du) * (1.0f - g.dv);
                 float w01 = (1.0f - g.du) * g.dv;

@@ -135,12 +135,13 @@ void raise_on(int rc, const char *what) {
 
 // Same positional order as the reference's flash_bevpool_forward
 // (flashbev/flashbevpool/src/flash_bevpool.cpp:79-101).  The four kernel-variant booleans
-// select nothing here (one kernel serves all); the trailing arguments are extensions.
+// select nothing here (one kernel serves all); the trailing arguments are extensions.  The six voxel
+// scalars are float64 (the reference takes them as float): cell centres are evaluated in float64.
 void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &image_feats,
                            const at::Tensor &projection_matrices, const at::Tensor &feature_size,
-                           const at::Tensor &image_size, const at::Tensor &grid_size, float voxel_size_x,
-                           float voxel_size_y, float voxel_size_z, float voxel_x_min, float voxel_y_min,
-                           float voxel_z_min, at::Tensor out, int64_t total_threads, int depth_distribution,
+                           const at::Tensor &image_size, const at::Tensor &grid_size, double voxel_size_x,
+                           double voxel_size_y, double voxel_size_z, double voxel_x_min, double voxel_y_min,
+                           double voxel_z_min, at::Tensor out, int64_t total_threads, int depth_distribution,
                            bool use_shared_memory, bool optimize_z_precompute, bool use_warp_kernel,
                            bool use_vectorized_load, float epsilon, float depth_weight_threshold,
                            float depth_min, float depth_step, int reduction, std::optional<at::Tensor> count_out) {
@@ -186,9 +187,9 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
     auto roi = host_floats(roi_range, 6, "roi_range");
     const int32_t g[3] = {p.grid_x, p.grid_y, p.grid_z};
     for (int a = 0; a < 3; ++a) {
-        p.voxel_min[a] = roi[2 * a];
-        volatile float extent = roi[2 * a + 1] - roi[2 * a];   // one rounded fp32 subtraction
-        p.voxel_size[a] = extent / (float)g[a];                // one rounded fp32 division
+        // float64 arithmetic on the fp32 bounds, exactly what the Python operator hands the forward
+        p.voxel_min[a] = (double)roi[2 * a];
+        p.voxel_size[a] = ((double)roi[2 * a + 1] - (double)roi[2 * a]) / (double)g[a];
     }
     check_dev(out_grad, depth_params, "out_grad");
     TORCH_CHECK(out_grad.scalar_type() == at::kFloat, "flashbevpool_ext: out_grad must be float32");
@@ -280,7 +281,7 @@ std::vector<at::Tensor> sample_geometry(const at::Tensor &projection_matrices, i
     p.feat_h = (int32_t)feat_h; p.feat_w = (int32_t)feat_w;
     p.image_h = (int32_t)image_h; p.image_w = (int32_t)image_w;
     p.grid_x = (int32_t)grid_size[0]; p.grid_y = (int32_t)grid_size[1]; p.grid_z = (int32_t)grid_size[2];
-    for (int a = 0; a < 3; ++a) { p.voxel_min[a] = (float)voxel_min[a]; p.voxel_size[a] = (float)voxel_size[a]; }
+    for (int a = 0; a < 3; ++a) { p.voxel_min[a] = voxel_min[a]; p.voxel_size[a] = voxel_size[a]; }
     p.epsilon = epsilon;
     p.channels = 1; p.depth_bins = 2;
     p.proj_stride = (int32_t)(projection_matrices.size(2) * 4);

@@ -87,10 +87,12 @@ def _host_values(x, n: int, name: str):
 
 
 def voxel_geometry(roi_range: Sequence[float], grid_size: Sequence[int]):
-    """(voxel_min[3], voxel_size[3]) as fp32 values: size = (max - min) / grid, one rounded
-    fp32 subtraction and one rounded fp32 division (flash_bevpool.py:62-67)."""
-    r = np.asarray(roi_range, dtype=np.float32)
-    g = np.asarray(grid_size, dtype=np.float32)
+    """(voxel_min[3], voxel_size[3]) in float64: the bounds are the fp32 values of ``roi_range``
+    (what the reference's float tensor holds, flash_bevpool.py:52), the size is
+    (max - min) / grid evaluated in float64 on them.  The kernels round each cell centre
+    min + (i + 0.5) * size once, to fp32."""
+    r = np.asarray(roi_range, dtype=np.float32).astype(np.float64)
+    g = np.asarray(grid_size, dtype=np.float64)
     size = (r[1::2] - r[0::2]) / g
     return [float(v) for v in r[0::2]], [float(v) for v in size]
 

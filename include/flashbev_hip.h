@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 4
+#define FBEV_ABI_VERSION 5
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -58,9 +58,15 @@ typedef struct fbev_problem {
     int32_t grid_x;      /* BEV cells along x */
     int32_t grid_y;
     int32_t grid_z;      /* height bins reduced per cell */
-    float voxel_min[3];  /* lower edge of the region of interest along x, y, z */
-    float voxel_size[3]; /* cell size along x, y, z: (max - min) / grid, an fp32 division;
-                            cell i has its centre at min + (i + 0.5) * size */
+    double voxel_min[3];  /* lower edge of the region of interest along x, y, z (the reference's
+                             voxel_x_min .. voxel_z_min, flash_bevpool.py:65-67, widened) */
+    double voxel_size[3]; /* cell size along x, y, z: (max - min) / grid in float64 (the reference's
+                             voxel_size_x .. voxel_size_z, flash_bevpool.py:62-64, widened).  Cell i has
+                             its centre at fp32(min + (i + 0.5) * size), evaluated in float64 and
+                             rounded once: the correctly rounded centre, within an ulp of the dense
+                             path's linspace(min, max, grid + 1)[:-1] + size / 2
+                             (sampling_vt.py:364-378).  An fp32 size would carry its rounding error
+                             i times along the axis. */
     float epsilon;       /* added to sigma; lower clamp of the perspective divisor */
     float depth_weight_threshold; /* samples with weight < threshold are dropped */
     int32_t depth_distribution;   /* FBEV_GAUSSIAN / FBEV_LAPLACE / FBEV_CATEGORICAL */

@@ -92,11 +92,18 @@ static inline void project_sample(const oracle_problem *p, const float *P,
     g->valid = 1;
 }
 
-static inline void voxel_sizes(const oracle_problem *p, float *vx, float *vy, float *vz)
+/*
+ * Centre of cell i along one axis: the float64 value lo + (i + 0.5) * (hi - lo) / n, rounded once
+ * to fp32 (the roi bounds are fp32 values, widened exactly).  The reference's dense path takes
+ * linspace(lo, hi, n + 1)[:-1] + step / 2 (sampling_vt.py:364-378), its fused kernel
+ * lo + (i + 0.5) * fp32(step) (flash_bevpool_cuda.cu:45-46); the second accumulates the rounding
+ * of the fp32 step along the axis (0.8 m is not an fp32 number), which a Gaussian tail weight
+ * magnifies beyond the parity tolerance, so the correctly rounded centre is the canonical one.
+ */
+static inline float voxel_centre(float lo, float hi, int n, int i)
 {
-    *vx = (p->roi[1] - p->roi[0]) / (float)p->gx;
-    *vy = (p->roi[3] - p->roi[2]) / (float)p->gy;
-    *vz = (p->roi[5] - p->roi[4]) / (float)p->gz;
+    double step = ((double)hi - (double)lo) / (double)n;
+    return (float)((double)lo + ((double)i + 0.5) * step);
 }
 
 static inline float bilerp(const sample_geom *g, float a00, float a01, float a10, float a11)
@@ -159,17 +166,15 @@ static inline void eval_depth(const oracle_problem *p, const float *depth,
 void fbev_oracle_geometry(const oracle_problem *p, const float *proj /* [B,N,12] */,
                           uint8_t *mask, int32_t *idx, float *frac, float *depth_out)
 {
-    float vx, vy, vz;
-    voxel_sizes(p, &vx, &vy, &vz);
     size_t s = 0;
     for (int b = 0; b < p->B; ++b)
         for (int iy = 0; iy < p->gy; ++iy)
             for (int ix = 0; ix < p->gx; ++ix) {
-                float x = p->roi[0] + ((float)ix + 0.5f) * vx;
-                float y = p->roi[2] + ((float)iy + 0.5f) * vy;
+                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix);
+                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy);
                 for (int n = 0; n < p->N; ++n)
                     for (int iz = 0; iz < p->gz; ++iz, ++s) {
-                        float z = p->roi[4] + ((float)iz + 0.5f) * vz;
+                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz);
                         sample_geom g;
                         project_sample(p, proj + ((size_t)b * p->N + n) * 12, x, y, z, &g);
                         if (mask) mask[s] = (uint8_t)g.valid;
@@ -196,16 +201,14 @@ void fbev_oracle_geometry(const oracle_problem *p, const float *proj /* [B,N,12]
 void fbev_oracle_forward(const oracle_problem *p, const float *depth, const float *feats,
                          const float *proj, float *out, float *count, uint8_t *keep)
 {
-    float vx, vy, vz;
-    voxel_sizes(p, &vx, &vy, &vz);
     const int C = p->C, H = p->H, W = p->W;
     float *acc = (float *)malloc(sizeof(float) * (size_t)C);
     size_t s = 0;
     for (int b = 0; b < p->B; ++b)
         for (int iy = 0; iy < p->gy; ++iy)
             for (int ix = 0; ix < p->gx; ++ix) {
-                float x = p->roi[0] + ((float)ix + 0.5f) * vx;
-                float y = p->roi[2] + ((float)iy + 0.5f) * vy;
+                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix);
+                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy);
                 for (int c = 0; c < C; ++c) acc[c] = 0.0f;
                 float cnt = 0.0f;
                 for (int n = 0; n < p->N; ++n) {
@@ -213,7 +216,7 @@ void fbev_oracle_forward(const oracle_problem *p, const float *depth, const floa
                     const float *dcam = depth + cam * H * W * p->D;
                     const float *fcam = feats + cam * H * W * C;
                     for (int iz = 0; iz < p->gz; ++iz, ++s) {
-                        float z = p->roi[4] + ((float)iz + 0.5f) * vz;
+                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz);
                         sample_geom g;
                         if (keep) keep[s] = 0;
                         project_sample(p, proj + cam * 12, x, y, z, &g);
@@ -249,8 +252,6 @@ void fbev_oracle_forward(const oracle_problem *p, const float *depth, const floa
 void fbev_oracle_backward(const oracle_problem *p, const float *grad_out, const float *depth,
                           const float *feats, const float *proj, float *d_depth, float *d_feats)
 {
-    float vx, vy, vz;
-    voxel_sizes(p, &vx, &vy, &vz);
     const int C = p->C, H = p->H, W = p->W, Dd = p->D, NZ = p->N * p->gz;
     size_t n_feat = (size_t)p->B * p->N * H * W * C;
     size_t n_dep = (size_t)p->B * p->N * H * W * Dd;
@@ -261,14 +262,14 @@ void fbev_oracle_backward(const oracle_problem *p, const float *grad_out, const 
     for (int b = 0; b < p->B; ++b)
         for (int iy = 0; iy < p->gy; ++iy)
             for (int ix = 0; ix < p->gx; ++ix) {
-                float x = p->roi[0] + ((float)ix + 0.5f) * vx;
-                float y = p->roi[2] + ((float)iy + 0.5f) * vy;
+                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix);
+                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy);
                 int cnt = 0;
                 for (int n = 0; n < p->N; ++n) {
                     size_t cam = (size_t)b * p->N + n;
                     for (int iz = 0; iz < p->gz; ++iz) {
                         int k = n * p->gz + iz;
-                        float z = p->roi[4] + ((float)iz + 0.5f) * vz;
+                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz);
                         project_sample(p, proj + cam * 12, x, y, z, &gs[k]);
                         es[k].keep = 0;
                         if (!gs[k].valid) continue;

@@ -90,8 +90,8 @@ def test_backward_single_gradient():
 
 @pytest.mark.parametrize("dist", [0, 1])
 def test_forward_backward_vs_dense_torch(dist):
-    """The named parity target: the dense grid_sample path in fp32, with its own distance to a
-    float64 evaluation as the yardstick for the ill-conditioned elements."""
+    """The named parity target: the dense grid_sample path in fp32 at rtol 1e-4 / atol 1e-5, with
+    its own distance to a float64 evaluation as the allowance for the ill-conditioned elements."""
     w, x = _inputs("cfg2_surround", dist)
     kw = U.op_kwargs(w, dist)
     cpu = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in x.items()}
@@ -110,10 +110,16 @@ def test_forward_backward_vs_dense_torch(dist):
         print(f"{what}: vs dense fp32 bad={bad} max={maxabs:.3e} ratio={ratio:.1f} | dense fp32 vs fp64 "
               f"bad={floor_bad} max={floor_abs:.3e} ratio={floor_ratio:.1f} | ours vs fp64 bad={ours_bad} "
               f"max={ours_abs:.3e} ratio={ours_ratio:.1f}")
-        # two fp32 formulations of an ill-conditioned function (a Gaussian tail weight has
-        # relative condition number z^2 up to ~27): a few elements leave the band in both
-        assert bad <= 2e-2 * got.numel()
-        assert ours_ratio <= 4.0 * max(floor_ratio, 1.0)
+        # The stated tolerance (rtol 1e-4, atol 1e-5).  A Gaussian tail weight has relative condition
+        # number z^2 up to ~27, so the dense fp32 path itself leaves that band against its own float64
+        # evaluation on a few elements (`floor_bad`; observed at this workload: Gaussian out 2,
+        # d_feats 24, d_depth 54; Laplace 0, 0, 13).  The kernels may leave it on no more elements
+        # than that plus a handful, against the fp32 path and against float64 alike.
+        assert bad <= floor_bad + 8, (what, bad, floor_bad)
+        assert ours_bad <= floor_bad + 8, (what, ours_bad, floor_bad)
+        assert ours_ratio <= 1.5 * max(floor_ratio, 1.0), (what, ours_ratio, floor_ratio)
+        if dist == 1 and what == "out":
+            assert bad == 0 and ours_bad == 0, (what, bad, ours_bad)
         if what == "out":
             # the reference's own (forward-only) acceptance statistics, tools/profile_differences.py:70-106
             m = U.reference_metrics(got.numpy(), r32.numpy())

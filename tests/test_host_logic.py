@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in flashbev_hip.h but not exported"
     assert sorted(capi.EXPORTS) == names
-    assert lib.fbev_abi_version() == 4
+    assert lib.fbev_abi_version() == 5
     assert lib.fbev_problem_size() == ctypes.sizeof(capi.FbevProblem)
 
 
@@ -42,7 +42,7 @@ def test_header_struct_matches_binding():
     text = open(os.path.join(ROOT, "include", "flashbev_hip.h")).read()
     body = re.search(r"typedef struct fbev_problem \{(.*?)\} fbev_problem;", text, flags=re.S).group(1)
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
-    fields = re.findall(r"(?:int32_t|float)\s+([a-z_]+)(?:\[\d\])?;", body)
+    fields = re.findall(r"(?:int32_t|float|double)\s+([a-z_]+)(?:\[\d\])?;", body)
     assert fields == [f[0] for f in capi.FbevProblem._fields_]
 
 
@@ -137,12 +137,19 @@ def test_workload_generator_shapes_and_seeding():
     assert not torch.equal(p4[0], p4[1])
 
 
-def test_voxel_geometry_is_fp32_arithmetic():
+def test_voxel_geometry_is_float64_arithmetic_on_the_fp32_bounds():
     vmin, vsize = voxel_geometry((-51.2, 51.2, -51.2, 51.2, -5.0, 3.0), (200, 200, 12))
-    r = np.float32([-51.2, 51.2, -5.0, 3.0])
-    assert vsize[0] == float((r[1] - r[0]) / np.float32(200))
-    assert vsize[2] == float((r[3] - r[2]) / np.float32(12))
+    r = np.float32([-51.2, 51.2, -5.0, 3.0]).astype(np.float64)
+    assert vsize[0] == (r[1] - r[0]) / 200.0 and vsize[2] == (r[3] - r[2]) / 12.0
     assert vmin == [float(r[0]), float(r[0]), float(r[2])]
+    # the centres the kernels form from these stay within two ulps (of the bound's magnitude) of the
+    # dense path's linspace(lo, hi, n + 1)[:-1] + step / 2 (sampling_vt.py:364-378), all along the axis
+    import torch
+    lo, hi, n = -51.2, 51.2, 200
+    edges = torch.linspace(lo, hi, n + 1)
+    dense = (edges[:-1] + (edges[1] - edges[0]) / 2).numpy()
+    mine = (vmin[0] + (np.arange(n) + 0.5) * vsize[0]).astype(np.float32)
+    assert np.all(np.abs(mine.astype(np.float64) - dense) <= 2 * np.spacing(np.float32(hi)))
 
 
 class FakeExt:
