@@ -78,6 +78,27 @@ def have_libs() -> bool:
     return os.path.exists(HIP_LIB) and os.path.exists(EXT_LIB)
 
 
+def stale() -> bool:
+    """True when a source under csrc/ or the public header is newer than a built library.  Where the
+    sources do not travel with the libraries (no csrc/ directory) nothing is stale."""
+    if not have_libs() or not os.path.isdir(CSRC):
+        return False
+    built = min(os.path.getmtime(HIP_LIB), os.path.getmtime(EXT_LIB))
+    srcs = [os.path.join(CSRC, f) for f in os.listdir(CSRC)] + [os.path.join(INCLUDE, "flashbev_hip.h")]
+    return any(os.path.exists(f) and os.path.getmtime(f) > built for f in srcs)
+
+
+def header_abi_version():
+    """FBEV_ABI_VERSION as include/flashbev_hip.h declares it (None without the header)."""
+    import re
+    try:
+        text = open(os.path.join(INCLUDE, "flashbev_hip.h")).read()
+    except OSError:
+        return None
+    m = re.search(r"#define\s+FBEV_ABI_VERSION\s+(\d+)", text)
+    return int(m.group(1)) if m else None
+
+
 if __name__ == "__main__":
     build_all()
     sys.exit(0)

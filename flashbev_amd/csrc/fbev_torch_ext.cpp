@@ -98,15 +98,18 @@ fbev_problem describe(const at::Tensor &depth, const at::Tensor &feats, const at
     p.depth_bins = (int32_t)depth.size(4);
     p.in_dtype = dtype_code(feats, "image_feats");
 
-    // feature_size [B,N,2] repeats (H, W) of the feature tensor for every camera; it can be
-    // checked for free only when it already lives on the host.
+    // feature_size [B,N,2] must repeat (H, W) of the feature tensor for every camera.  The reference
+    // kernel reads it per camera (flash_bevpool_cuda.cu:134-135); valid sizes smaller than a padded
+    // tensor are not supported here, so it is always checked (a device tensor costs one synchronous
+    // copy, like the reference's read of grid_size; the Python operator passes a host table).
     TORCH_CHECK(feature_size.numel() == (int64_t)p.batch * p.num_cams * 2,
                 "flashbevpool_ext: feature_size must be [B,N,2], got ", feature_size.sizes());
-    if (!feature_size.is_cuda()) {
+    {
         auto fs = host_ints(feature_size, feature_size.numel(), "feature_size");
         for (size_t i = 0; i < fs.size(); i += 2)
             TORCH_CHECK(fs[i] == p.feat_h && fs[i + 1] == p.feat_w, "flashbevpool_ext: feature_size entry (",
-                        fs[i], ",", fs[i + 1], ") differs from the feature tensor's (", p.feat_h, ",", p.feat_w, ")");
+                        fs[i], ",", fs[i + 1], ") differs from the feature tensor's (", p.feat_h, ",", p.feat_w,
+                        "); per-camera valid sizes are not supported");
     }
     auto im = host_ints(image_size, 2, "image_size");
     auto gs = host_ints(grid_size, 3, "grid_size");
@@ -240,6 +243,10 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
     // pair_capacity selects the exactly packed layout (what does not fit is applied with atomics).
     auto run_gather = [&]() -> int {
         const uint64_t max_pairs = fbev_backward_max_pairs(&p);
+        // pair positions and claim counters are 32-bit in the library: say so before any allocation
+        // (what fbev_backward_gather itself would answer), so that "auto" can still take the column owner
+        const uint64_t texels = (uint64_t)p.batch * p.num_cams * p.feat_h * p.feat_w;
+        if (max_pairs == 0 || max_pairs >= (1ull << 31) || texels * 32 >= (1ull << 31)) return FBEV_ERR_TOO_LARGE;
         uint64_t cap = pair_capacity >= 0 ? (uint64_t)pair_capacity : max_pairs;
         if (cap > max_pairs) cap = max_pairs;
         const size_t bytes = fbev_backward_workspace_bytes(&p, cap);

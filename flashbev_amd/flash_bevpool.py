@@ -59,31 +59,59 @@ def _pair_capacity(batch: int, cams: int, grid) -> int:
     return max(0, int(limit_mb * 2 ** 20) // 32)
 
 
-_host_cache: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()
+# id(tensor) -> (weak reference, version, values).  Keyed by identity: a mapping keyed by the
+# tensors themselves would compare them with ``==`` on lookup, which is elementwise.
+_host_cache: dict = {}
+
+
+def _device_values(x):
+    """Values of a small device tensor, read once per tensor object and version (one synchronous
+    copy), so that a tensor reused across calls (a registered buffer, say) costs nothing later."""
+    key = id(x)
+    hit = _host_cache.get(key)
+    if hit is not None and hit[0]() is x and hit[1] == x._version:
+        return hit[2]
+    vals = x.detach().reshape(-1).tolist()
+    ref = weakref.ref(x, lambda _r, key=key: _host_cache.pop(key, None))
+    _host_cache[key] = (ref, x._version, vals)
+    return vals
 
 
 def _host_values(x, n: int, name: str):
-    """Values of a small size/range argument as Python numbers.
-
-    Sequences and CPU tensors cost nothing.  A device tensor costs one synchronous copy,
-    remembered per tensor object and version so that a tensor reused across calls (a
-    registered buffer, say) is read once.
-    """
+    """Values of a small size/range argument as Python numbers.  Sequences and CPU tensors cost
+    nothing; a device tensor costs one synchronous copy the first time it is seen."""
     if isinstance(x, torch.Tensor):
         if x.numel() != n:
             raise ValueError(f"{name} must have {n} elements, got shape {tuple(x.shape)}")
         if x.device.type == "cpu":
             return x.reshape(-1).tolist()
-        hit = _host_cache.get(x)
-        if hit is not None and hit[0] == x._version:
-            return hit[1]
-        vals = x.detach().reshape(-1).tolist()
-        _host_cache[x] = (x._version, vals)
-        return vals
+        return _device_values(x)
     vals = list(x)
     if len(vals) != n:
         raise ValueError(f"{name} must have {n} elements, got {len(vals)}")
     return vals
+
+
+def _check_feature_size(feature_size, cameras: int, H: int, W: int):
+    """``feature_size`` must repeat the feature tensor's (H, W) for every camera.  The reference
+    kernel reads it per camera (flash_bevpool_cuda.cu:134-135), so a caller could pass valid sizes
+    smaller than a padded tensor; that is not supported here and raises instead of silently
+    sampling the padding.  ``None`` is accepted (the shape is used)."""
+    if feature_size is None:
+        return
+    if isinstance(feature_size, torch.Tensor):
+        if feature_size.numel() != 2 * cameras:
+            raise ValueError(f"feature_size must have shape [B, N, 2] = {2 * cameras} elements, got "
+                             f"{tuple(feature_size.shape)}")
+        vals = (feature_size.reshape(-1).tolist() if feature_size.device.type == "cpu"
+                else _device_values(feature_size))
+    else:
+        vals = [int(v) for row in feature_size for v in (row if hasattr(row, "__iter__") else [row])]
+        if len(vals) != 2 * cameras:
+            raise ValueError(f"feature_size must hold (H, W) for each of {cameras} cameras")
+    if any(int(vals[i]) != (H, W)[i & 1] for i in range(len(vals))):
+        raise RuntimeError(f"feature_size must equal the feature maps' shape (H, W) = ({H}, {W}) for every "
+                         f"camera; per-camera valid sizes inside a padded tensor are not supported")
 
 
 def voxel_geometry(roi_range: Sequence[float], grid_size: Sequence[int]):
@@ -146,12 +174,10 @@ class FlashBEVPool(torch.autograd.Function):
         roi = tuple(float(v) for v in _host_values(roi_range, 6, "roi_range"))
         image_t, grid_t, roi_t, vmin, vsize = _host_arguments(grid, image, roi)
 
-        # feature_size repeats the feature tensor's (H, W) per camera; hand the extension a
-        # host copy built from the shape unless the caller already gave a host tensor.
-        if isinstance(feature_size, torch.Tensor) and feature_size.device.type == "cpu":
-            fs_host = feature_size.to(torch.int32).contiguous()
-        else:
-            fs_host = _feature_size_table(B * N, H, W)
+        # feature_size repeats the feature tensor's (H, W) per camera: checked (a device tensor is
+        # read once per object), then the extension gets a host table built from the shape
+        _check_feature_size(feature_size, B * N, H, W)
+        fs_host = _feature_size_table(B * N, H, W)
 
         out = torch.empty((B, grid[1], grid[0], C), dtype=torch.float32, device=image_feats.device)
         red = 0 if reduction == "mean" else 1

@@ -174,6 +174,29 @@ def test_operator_errors_on_gpu():
     out = flash_bevpool(**dict(base, image_size=x["image_size"].cuda(), roi_range=x["roi_range"].cuda(),
                                grid_size=x["grid_size"].cuda(), feature_size=x["feature_size"].cuda()))
     assert torch.equal(out, flash_bevpool(**base))
+    with pytest.raises(RuntimeError, match="feature_size"):
+        flash_bevpool(**dict(base, feature_size=torch.tensor([8, 22], dtype=torch.int32).repeat(1, 6, 1).cuda()))
+
+
+def test_device_resident_size_tensors_are_reused_across_calls():
+    """A module keeps grid_size / image_size / roi_range as registered buffers and passes the same
+    device tensors on every call: they are read once per object and version, and an in-place edit
+    is seen."""
+    w = small(channels=16, grid_size=(16, 16, 2))
+    x = make_inputs(w, "parametric", device="cuda")
+    dev = {k: x[k].cuda() for k in ("image_size", "roi_range", "grid_size", "feature_size")}
+    args = dict(image_feats=x["image_feats"], depth_params=x["depth_params"], projection_matrices=x["projection_matrices"])
+    want = flash_bevpool(**args, **{k: x[k] for k in dev})
+    for _ in range(3):
+        assert torch.equal(flash_bevpool(**args, **dev), want)
+    dev["grid_size"][2] = 4                                   # in place: same object, new version
+    want4 = flash_bevpool(**args, **dict({k: x[k] for k in dev}, grid_size=(16, 16, 4)))
+    assert torch.equal(flash_bevpool(**args, **dev), want4) and not torch.equal(want4, want)
+    dev["roi_range"][5] += 1.0
+    roi = x["roi_range"].clone()
+    roi[5] += 1.0
+    want5 = flash_bevpool(**args, **dict({k: x[k] for k in dev}, grid_size=(16, 16, 4), roi_range=roi))
+    assert torch.equal(flash_bevpool(**args, **dev), want5)
 
 
 def test_results_are_reproducible_and_stream_ordered():
