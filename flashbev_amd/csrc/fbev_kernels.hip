@@ -325,6 +325,141 @@ int check_backward_args(const fbev_problem *p, const float *grad_out, const void
     return FBEV_OK;
 }
 
+
+// ---------------------------------------------------------------- library-owned scratch
+// Workspace of fbev_backward_gather_static, for callers that cannot allocate: one array per
+// GPU, held from the moment the library is loaded there until the process ends.  In host code
+// the array's name is a stand-in, not a device address; the address on each device comes from
+// hipGetSymbolAddress, once per device, and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[FBEV_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mu;
+void *scratch_ptr[kMaxDevices] = {};
+
+int scratch_of_current_device(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FBEV_ERR_LAUNCH;
+    std::lock_guard<std::mutex> g(scratch_mu);
+    if (scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return FBEV_ERR_LAUNCH;
+        scratch_ptr[dev] = ptr;
+    }
+    *out = scratch_ptr[dev];
+    return FBEV_OK;
+}
+
+int backward_gather_impl(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                         const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    int rc = validate(p, true);
+    if (rc != FBEV_OK) return rc;
+    rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
+    if (rc != FBEV_OK) return rc;
+    if (!d_depth && !d_feats) return FBEV_OK;
+    if (!workspace) return FBEV_ERR_NULL;
+    if ((uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
+    const size_t index_bytes = ws_index_bytes(p);
+    if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
+    // pair positions are 32-bit: every sample must be countable
+    if (sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    // the texel pass addresses grad_out rows in 32-bit units (16 bytes, or one float off the vector path)
+    const bool rows_vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
+    if ((long long)p->batch * p->grid_y * p->grid_x * (rows_vec4 ? p->channels / 4 : p->channels) >= (1ll << 32))
+        return FBEV_ERR_TOO_LARGE;
+    size_t cap64 = (workspace_bytes - index_bytes) / sizeof(Pair);
+    const int cap = cap64 > 0x7fffffffull ? 0x7fffffff : (int)cap64;
+    Plan pl;
+    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl, kCellPassWaves);
+    if (rc != FBEV_OK) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int *cursor = static_cast<int *>(workspace);
+    Pair *pairs = reinterpret_cast<Pair *>(static_cast<char *>(workspace) + index_bytes);
+    const long long texels = texel_count(p);
+    const long long counters = counter_count(p), chunks = chunk_count(p);
+    int *chunk_prefix = cursor + counters;
+
+    // A workspace with room for every sample gets fixed segments: each (texel, replica)
+    // owns cap / (texels * kFixedReplicas) pair slots, and the counting pass and the prefix sums
+    // are not needed.  (A texel that outgrows its segments falls back to atomics, like a full
+    // pair array does.)  Smaller workspaces are packed exactly: count, scan, fill.
+    const bool fixed = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (texels * kFixedReplicas) >= kFixedMinSegment;
+    const int seg_cap = fixed ? (int)(cap / (texels * kFixedReplicas)) : 0;
+    rc = launch_zero(cursor, fixed ? texels * kFixedReplicas : counters, accumulate ? nullptr : d_depth,
+                     texels * p->depth_bins, accumulate ? nullptr : d_feats, texels * p->channels, st);
+    if (rc != FBEV_OK) return rc;
+    if (!fixed) {
+        switch (p->in_dtype) {
+            case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, st); break;
+            case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, st); break;
+            default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, st); break;
+        }
+        if (rc != FBEV_OK) return rc;
+        {
+            prof::Scope timer(prof::kScanChunks, st);
+            hipLaunchKernelGGL(fbev_scan_chunks_kernel, dim3((unsigned)chunks), dim3(1024), 0, st, cursor, counters,
+                               chunk_prefix);
+        }
+        if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+        {
+            prof::Scope timer(prof::kScanSums, st);
+            hipLaunchKernelGGL(fbev_scan_sums_kernel, dim3(1), dim3(1024), 0, st, chunk_prefix, (int)chunks);
+        }
+        if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+    }
+    const int *prefix_arg = fixed ? nullptr : chunk_prefix;
+    const int cap_arg = fixed ? seg_cap : cap;
+    // samples a claim counter gets if every sample is kept
+    const bool claim_runs = sample_count(p) / (fixed ? texels * kFixedReplicas : counters) >= kClaimRunsFrom;
+    rc = claim_runs ? dispatch_cells<2>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
+                                        cap_arg, st)
+                    : dispatch_cells<1>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
+                                        cap_arg, st);
+    if (rc != FBEV_OK) return rc;
+
+    // texel pass: rows of grad_out are fp32, so 128-bit gathers need C % 4 == 0 and aligned rows
+    const bool vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
+    const int vec = vec4 ? 4 : 1;
+    const int cq = (p->channels + vec - 1) / vec;
+    const int lpr = cq < kWave ? cq : kWave;
+    // One, two or four wavefronts per texel.  A texel's block is a chain of dependent loads (list bounds,
+    // pairs, grad_out rows); small blocks fit the machine in fewer generations, large ones shorten the
+    // chain of a long list.  What is known here is only how many samples a texel could get if every one were
+    // kept.  Measured (us for 1 / 2 / 4 wavefronts; Laplace, then the categorical model, which keeps twice
+    // as many): 23 possible samples per texel 8 / 9 / 11; 186 per texel and 4224 texels 20 / 19 / 23 and
+    // 39 / 30 / 31; 186 per texel and 67 584 texels 125 / 154 / 239 and 256 / 274 / 365; 454 per texel
+    // 38 / 29 / 29 and 80 / 60 / 52; 909 per texel 493 / 426 / 431; 2727 per texel 352 / 209 / 124.
+    const uint64_t per_texel = fbev_backward_max_pairs(p) / (uint64_t)texels;
+    const int texel_waves = (per_texel < kTexelOneWaveBelow || (texels >= kTexelManyTexels && per_texel < 3 * kTexelOneWaveBelow)) ? 1
+                            : (per_texel < kTexelTwoWavesBelow ? 2 : kWavesPerBlock);
+    const int nw = (kWave / lpr) * texel_waves;
+    // the depth gradient rides on the pairs exactly when the cell pass folds it in (one channel pass
+    // and room for the depth bin in a pair's first word)
+    const int from_pairs =
+        (d_depth != nullptr && pl.k.C <= pl.k.lanes_per_slot * pl.vec * pl.cpl && pl.k.bin_bits >= 0) ? 1 : 0;
+    const size_t lds = ((size_t)texel_waves * kWave * 2 + (size_t)nw * (lpr * vec + 2) +
+                        (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) * sizeof(float);
+    long long want_split = kTexelSplitBelow / texels;
+    const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
+    prof::Scope timer(prof::kBackwardTexel, st);
+    const dim3 tgrid((unsigned)texels, n_split), tblock(kWave * texel_waves);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats,
+                           lpr, from_pairs, accumulate ? 0 : 1);
+    };
+    if (vec4) {
+        if (texel_waves == 1) launch(fbev_backward_texel_kernel<4, 1>);
+        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<4, 2>);
+        else launch(fbev_backward_texel_kernel<4, kWavesPerBlock>);
+    } else {
+        if (texel_waves == 1) launch(fbev_backward_texel_kernel<1, 1>);
+        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<1, 2>);
+        else launch(fbev_backward_texel_kernel<1, kWavesPerBlock>);
+    }
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
 }  // namespace
 
 extern "C" {
@@ -434,112 +569,28 @@ size_t fbev_backward_workspace_bytes(const fbev_problem *p, uint64_t pair_capaci
 int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
                          const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
                          size_t workspace_bytes, void *stream) {
+    return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
+                                workspace_bytes, stream);
+}
+
+int fbev_backward_gather_static(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                                const float *proj, float *d_depth, float *d_feats, int accumulate, void *stream) {
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
-    rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
-    if (rc != FBEV_OK) return rc;
-    if (!d_depth && !d_feats) return FBEV_OK;
-    if (!workspace) return FBEV_ERR_NULL;
-    if ((uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
-    const size_t index_bytes = ws_index_bytes(p);
-    if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
-    // pair positions are 32-bit: every sample must be countable
-    if (sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
-    // the texel pass addresses grad_out rows in 32-bit units (16 bytes, or one float off the vector path)
-    const bool rows_vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
-    if ((long long)p->batch * p->grid_y * p->grid_x * (rows_vec4 ? p->channels / 4 : p->channels) >= (1ll << 32))
+    // the per-kernel timers create HIP events: not in a call that promises to allocate nothing
+    if (prof::enabled.load(std::memory_order_relaxed)) return FBEV_ERR_UNSUPPORTED;
+    // fixed segments only (three launches): the scratch array must hold the worst case of one pair per sample
+    const uint64_t max_pairs = fbev_backward_max_pairs(p);
+    if (max_pairs >= (1ull << 31) || ws_index_bytes(p) + (size_t)max_pairs * sizeof(Pair) > (size_t)FBEV_STATIC_SCRATCH_BYTES)
         return FBEV_ERR_TOO_LARGE;
-    size_t cap64 = (workspace_bytes - index_bytes) / sizeof(Pair);
-    const int cap = cap64 > 0x7fffffffull ? 0x7fffffff : (int)cap64;
-    Plan pl;
-    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl, kCellPassWaves);
+    void *ws = nullptr;
+    rc = scratch_of_current_device(&ws);
     if (rc != FBEV_OK) return rc;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    int *cursor = static_cast<int *>(workspace);
-    Pair *pairs = reinterpret_cast<Pair *>(static_cast<char *>(workspace) + index_bytes);
-    const long long texels = texel_count(p);
-    const long long counters = counter_count(p), chunks = chunk_count(p);
-    int *chunk_prefix = cursor + counters;
-
-    // A workspace with room for every sample gets fixed segments: each (texel, replica)
-    // owns cap / (texels * kFixedReplicas) pair slots, and the counting pass and the prefix sums
-    // are not needed.  (A texel that outgrows its segments falls back to atomics, like a full
-    // pair array does.)  Smaller workspaces are packed exactly: count, scan, fill.
-    const bool fixed = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (texels * kFixedReplicas) >= kFixedMinSegment;
-    const int seg_cap = fixed ? (int)(cap / (texels * kFixedReplicas)) : 0;
-    rc = launch_zero(cursor, fixed ? texels * kFixedReplicas : counters, accumulate ? nullptr : d_depth,
-                     texels * p->depth_bins, accumulate ? nullptr : d_feats, texels * p->channels, st);
-    if (rc != FBEV_OK) return rc;
-    if (!fixed) {
-        switch (p->in_dtype) {
-            case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, st); break;
-            case FBEV_F16: rc = launch_count<__half>(pl, depth, proj, cursor, st); break;
-            default: rc = launch_count<bf16_raw>(pl, depth, proj, cursor, st); break;
-        }
-        if (rc != FBEV_OK) return rc;
-        {
-            prof::Scope timer(prof::kScanChunks, st);
-            hipLaunchKernelGGL(fbev_scan_chunks_kernel, dim3((unsigned)chunks), dim3(1024), 0, st, cursor, counters,
-                               chunk_prefix);
-        }
-        if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
-        {
-            prof::Scope timer(prof::kScanSums, st);
-            hipLaunchKernelGGL(fbev_scan_sums_kernel, dim3(1), dim3(1024), 0, st, chunk_prefix, (int)chunks);
-        }
-        if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
-    }
-    const int *prefix_arg = fixed ? nullptr : chunk_prefix;
-    const int cap_arg = fixed ? seg_cap : cap;
-    // samples a claim counter gets if every sample is kept
-    const bool claim_runs = sample_count(p) / (fixed ? texels * kFixedReplicas : counters) >= kClaimRunsFrom;
-    rc = claim_runs ? dispatch_cells<2>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
-                                        cap_arg, st)
-                    : dispatch_cells<1>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
-                                        cap_arg, st);
-    if (rc != FBEV_OK) return rc;
-
-    // texel pass: rows of grad_out are fp32, so 128-bit gathers need C % 4 == 0 and aligned rows
-    const bool vec4 = p->channels % 4 == 0 && (uintptr_t)grad_out % 16 == 0;
-    const int vec = vec4 ? 4 : 1;
-    const int cq = (p->channels + vec - 1) / vec;
-    const int lpr = cq < kWave ? cq : kWave;
-    // One, two or four wavefronts per texel.  A texel's block is a chain of dependent loads (list bounds,
-    // pairs, grad_out rows); small blocks fit the machine in fewer generations, large ones shorten the
-    // chain of a long list.  What is known here is only how many samples a texel could get if every one were
-    // kept.  Measured (us for 1 / 2 / 4 wavefronts; Laplace, then the categorical model, which keeps twice
-    // as many): 23 possible samples per texel 8 / 9 / 11; 186 per texel and 4224 texels 20 / 19 / 23 and
-    // 39 / 30 / 31; 186 per texel and 67 584 texels 125 / 154 / 239 and 256 / 274 / 365; 454 per texel
-    // 38 / 29 / 29 and 80 / 60 / 52; 909 per texel 493 / 426 / 431; 2727 per texel 352 / 209 / 124.
-    const uint64_t per_texel = fbev_backward_max_pairs(p) / (uint64_t)texels;
-    const int texel_waves = (per_texel < kTexelOneWaveBelow || (texels >= kTexelManyTexels && per_texel < 3 * kTexelOneWaveBelow)) ? 1
-                            : (per_texel < kTexelTwoWavesBelow ? 2 : kWavesPerBlock);
-    const int nw = (kWave / lpr) * texel_waves;
-    // the depth gradient rides on the pairs exactly when the cell pass folds it in (one channel pass
-    // and room for the depth bin in a pair's first word)
-    const int from_pairs =
-        (d_depth != nullptr && pl.k.C <= pl.k.lanes_per_slot * pl.vec * pl.cpl && pl.k.bin_bits >= 0) ? 1 : 0;
-    const size_t lds = ((size_t)texel_waves * kWave * 2 + (size_t)nw * (lpr * vec + 2) +
-                        (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) * sizeof(float);
-    long long want_split = kTexelSplitBelow / texels;
-    const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
-    prof::Scope timer(prof::kBackwardTexel, st);
-    const dim3 tgrid((unsigned)texels, n_split), tblock(kWave * texel_waves);
-    auto launch = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats,
-                           lpr, from_pairs, accumulate ? 0 : 1);
-    };
-    if (vec4) {
-        if (texel_waves == 1) launch(fbev_backward_texel_kernel<4, 1>);
-        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<4, 2>);
-        else launch(fbev_backward_texel_kernel<4, kWavesPerBlock>);
-    } else {
-        if (texel_waves == 1) launch(fbev_backward_texel_kernel<1, 1>);
-        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<1, 2>);
-        else launch(fbev_backward_texel_kernel<1, kWavesPerBlock>);
-    }
-    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+    return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, ws, (size_t)FBEV_STATIC_SCRATCH_BYTES,
+                                stream);
 }
+
+size_t fbev_static_scratch_bytes(void) { return (size_t)FBEV_STATIC_SCRATCH_BYTES; }
 
 int fbev_pillarpool_forward(const fbev_pillar_problem *p, const float *depth, const float *feats,
                             const float *u_coords, const float *v_coords, const float *z_coords,

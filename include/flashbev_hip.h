@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 5
+#define FBEV_ABI_VERSION 6
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -129,6 +129,28 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
 int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
                          const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
                          size_t workspace_bytes, void *stream);
+
+/*
+ * fbev_backward_gather without a workspace argument and without any allocation: the inverse map
+ * lives in a scratch array of FBEV_STATIC_SCRATCH_BYTES that the library itself holds in device
+ * memory (one copy per GPU, from the moment the library is loaded until the process ends).  It has
+ * no counterpart in the reference; it is for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call makes no
+ * hipMalloc / hipFree and calls no allocating library routine; inputs and outputs are the caller's,
+ * as in fbev_backward_gather, and the results are the same (fixed segments, three launches).
+ * Limits: the worst-case workspace, fbev_backward_workspace_bytes(p, fbev_backward_max_pairs(p)),
+ * must fit the scratch array, else FBEV_ERR_TOO_LARGE (128x128x8 cells x 6 cameras on a 16x44 map
+ * needs 25.8 MB); with the per-kernel timers enabled (fbev_profile_enable), which create events,
+ * it returns FBEV_ERR_UNSUPPORTED.  The device of `stream` must be the current device.  All calls
+ * on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered and each clears what it needs at its start.
+ */
+#define FBEV_STATIC_SCRATCH_BYTES (32u << 20)
+int fbev_backward_gather_static(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                                const float *proj, float *d_depth, float *d_feats, int accumulate, void *stream);
+
+/* FBEV_STATIC_SCRATCH_BYTES as the loaded library was built. */
+size_t fbev_static_scratch_bytes(void);
 
 /*
  * Backward by column ownership: the same gradients again, one launch, no global atomics and
