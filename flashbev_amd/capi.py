@@ -16,7 +16,8 @@ FBEV_GAUSSIAN, FBEV_LAPLACE, FBEV_CATEGORICAL = 0, 1, 2
 FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
 EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_gather_static",
-           "fbev_static_scratch_bytes", "fbev_backward_columns",
+           "fbev_static_scratch_bytes", "fbev_backward_persistent_workspace_bytes", "fbev_backward_workspace_init",
+           "fbev_backward_gather_persistent", "fbev_backward_columns",
            "fbev_backward_columns_workspace_bytes", "fbev_backward_max_pairs",
            "fbev_backward_workspace_bytes", "fbev_pillarpool_forward", "fbev_projection_matrices", "fbev_sample_geometry", "fbev_algorithmic_bytes",
            "fbev_profile_enable", "fbev_profile_kernel_count", "fbev_profile_kernel_name",
@@ -62,6 +63,12 @@ def load() -> ctypes.CDLL:
         lib.fbev_backward_gather_static.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp]
         lib.fbev_backward_gather_static.restype = ctypes.c_int
         lib.fbev_static_scratch_bytes.restype = ctypes.c_size_t
+        lib.fbev_backward_persistent_workspace_bytes.argtypes = [pp]
+        lib.fbev_backward_persistent_workspace_bytes.restype = ctypes.c_size_t
+        lib.fbev_backward_workspace_init.argtypes = [pp, vp, ctypes.c_size_t, vp]
+        lib.fbev_backward_workspace_init.restype = ctypes.c_int
+        lib.fbev_backward_gather_persistent.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp, ctypes.c_size_t, vp]
+        lib.fbev_backward_gather_persistent.restype = ctypes.c_int
         lib.fbev_backward_columns.argtypes = [pp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp, ctypes.c_size_t, vp]
         lib.fbev_backward_columns.restype = ctypes.c_int
         lib.fbev_backward_columns_workspace_bytes.argtypes = [pp]
@@ -160,6 +167,25 @@ def backward_gather_static(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, fe
     return load().fbev_backward_gather_static(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
                                               _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr),
                                               int(bool(accumulate)), _p(stream))
+
+
+def backward_persistent_workspace_bytes(p: FbevProblem) -> int:
+    return int(load().fbev_backward_persistent_workspace_bytes(ctypes.byref(p)))
+
+
+def backward_workspace_init(p: FbevProblem, workspace_ptr: int, workspace_bytes: int, stream: int = 0) -> int:
+    return load().fbev_backward_workspace_init(ctypes.byref(p), _p(workspace_ptr),
+                                               ctypes.c_size_t(int(workspace_bytes)), _p(stream))
+
+
+def backward_gather_persistent(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
+                               d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], workspace_ptr: int,
+                               workspace_bytes: int, stream: int = 0, accumulate: bool = True) -> int:
+    """fbev_backward_gather on a workspace prepared once by backward_workspace_init: two launches."""
+    return load().fbev_backward_gather_persistent(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
+                                                  _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr),
+                                                  int(bool(accumulate)), _p(workspace_ptr),
+                                                  ctypes.c_size_t(int(workspace_bytes)), _p(stream))
 
 
 def static_scratch_bytes() -> int:

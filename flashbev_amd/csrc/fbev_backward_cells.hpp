@@ -162,9 +162,17 @@ template <typename T, int VEC, int CPL, int FILL>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_kernel(
     KParams k, const float *__restrict__ grad_out, const T *__restrict__ depth, const T *__restrict__ feats,
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
-    const int *__restrict__ chunk_prefix, int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap) {
+    const int *__restrict__ chunk_prefix, int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap,
+    int *epoch, int set_stride) {
     extern __shared__ float4 smem[];
     constexpr int EF4 = 2;
+    if (FILL && epoch != nullptr) {
+        // persistent workspace: the call counter's low bit selects the set of claim counters, and the
+        // texel pass finds the counter where no block of its own writes (see struct Persist)
+        const int e = epoch[1];
+        cursor += (size_t)(e & 1) * set_stride;
+        if (blockIdx.x == 0 && threadIdx.x == 0) epoch[0] = e;
+    }
     // first corner texel and clamp flags of an entry
     auto entry_texel = [](const float4 &geo) { return FILL ? __float_as_int(geo.z) >> 2 : __float_as_int(geo.z); };
     auto entry_flags = [](const float4 &geo) { return FILL ? __float_as_int(geo.z) & 3 : __float_as_int(geo.w); };

@@ -22,11 +22,30 @@ constexpr int kTexelOneWaveBelow = 100;      // possible samples per texel below
 constexpr int kTexelManyTexels = 50000;      // ... or three times that when there are this many texels
 constexpr int kTexelTwoWavesBelow = 450;     // below which it is two wavefronts; four from there on
 constexpr int kTexelSegs = 4 * kFixedReplicas;   // lists of a texel with fixed segments: 4 first corners x replicas
+
+// What a persistent workspace adds to the fixed-segment layout, so that a call needs no zero-fill
+// launch (all null / 0 otherwise):
+//   epoch      two call counters.  The cell pass reads epoch[1] and copies it to epoch[0]; the texel
+//              pass reads epoch[0] and stores epoch[0] + 1 to epoch[1]: neither kernel reads a word
+//              that one of its own blocks writes.  The low bit selects the set of claim counters.
+//   sets       two sets of claim counters, set_stride ints apart.  A call claims in one set; its
+//              texel pass clears the other, which the previous call left behind and the next will use.
+//   ovf_*      gradient buffers of the workspace's own, all zero between calls.  What the cell pass
+//              cannot file (a full segment) or does not file (a depth gradient that does not ride on
+//              the pairs) it adds here with atomics; the texel pass of a texel that sees a full
+//              segment, the only texels such samples reach, takes its rows from here and clears them.
+struct Persist {
+    int *epoch;
+    int *sets;
+    int set_stride;
+    float *ovf_depth, *ovf_feats;
+};
+
 template <int VEC, int WAVES>
 __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
     const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
-    float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs, int fresh) {
+    float *__restrict__ d_feats, int lanes_per_row, int depth_from_pairs, int fresh, Persist ps) {
     extern __shared__ float4 smem[];
     // per wavefront 64 (grad_out row, coefficient) records of the chunk in hand, then the partial rows
     float2 *stage = reinterpret_cast<float2 *>(smem) + (threadIdx.x >> 6) * kWave;
@@ -47,6 +66,16 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     const int wave = threadIdx.x >> 6;
     constexpr int n_waves = WAVES;
     const bool counted = chunk_prefix != nullptr;
+    const bool persistent = ps.epoch != nullptr;
+    if (persistent) {
+        const int epoch = ps.epoch[0], set = epoch & 1;
+        seg_end = ps.sets + (size_t)set * ps.set_stride;
+        if (threadIdx.x == 0 && blockIdx.y == 0) {
+            // the counters of this texel in the set the next call claims in
+            *reinterpret_cast<int4 *>(ps.sets + (size_t)(set ^ 1) * ps.set_stride + (size_t)t * kFixedReplicas) = make_int4(0, 0, 0, 0);
+            if (blockIdx.x == 0) ps.epoch[1] = epoch + 1;
+        }
+    }
     // List e of the texel: first corner (e & 3 with fixed segments, e when counted): bit 0 = one
     // texel to the left, bit 1 = one row up; replica e >> 2 with fixed segments.  A cell's samples
     // on neighbouring height bins sit in different lists of the same replica, at about the same
@@ -91,13 +120,16 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
 #pragma unroll
     for (int j = 1; j < kTexelSegs; ++j) list_start[j] = __builtin_amdgcn_readlane(my_pre, j);
     const int n_all = __builtin_amdgcn_readlane(my_pre, kTexelSegs - 1) + __builtin_amdgcn_readlane(my_len, kTexelSegs - 1);
-    const int n_parts = min((int)gridDim.y, (n_all + 4 * kTexelPart - 1) / (4 * kTexelPart));
-    if ((int)blockIdx.y >= n_parts) return;      // uniform for the block (also when nothing was claimed)
+    // (a texel nothing was claimed for has no part at all, unless the workspace is persistent: then
+    // nobody has cleared the gradient buffers and its block stores the zeros)
+    const int n_parts = max(min((int)gridDim.y, (n_all + 4 * kTexelPart - 1) / (4 * kTexelPart)), persistent ? 1 : 0);
+    if ((int)blockIdx.y >= n_parts) return;      // uniform for the block
     const bool shared_texel = n_parts > 1;
     // The gradient buffers were cleared by this call (fresh) and nothing but this block touches the
     // texel unless a list spilled: then its rows are stored, not added, and the pass ends without a
     // dependent load.
-    const bool store_only = fresh != 0 && !shared_texel && __ballot(spilled) == 0ull;
+    const bool any_spill = __ballot(spilled) != 0ull;
+    const bool store_only = fresh != 0 && !shared_texel && !any_spill;
     const int part_lo = (int)(((long long)n_all * blockIdx.y) / n_parts);
     const int part_hi = (int)(((long long)n_all * (blockIdx.y + 1)) / n_parts);
     // the wavefronts take chunks of the sequence in turn: 64 pairs, fewer when that leaves a wavefront idle
@@ -255,16 +287,32 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             for (int w = 0; w < nw; ++w) sum += part[w * stride + c];
             if (d_feats != nullptr) {
                 float *dst = d_feats + (size_t)t * k.C + c0 + c;
-                if (shared_texel) atomic_add_f32(dst, sum);
+                if (persistent) {
+                    if (any_spill) {
+                        float *o = ps.ovf_feats + (size_t)t * k.C + c0 + c;
+                        sum += *o;
+                        *o = 0.0f;
+                    }
+                    if (fresh) *dst = sum;
+                    else *dst += sum;
+                } else if (shared_texel) atomic_add_f32(dst, sum);
                 else if (store_only) *dst = sum;
                 else *dst += sum;
             }
         }
         if (c0 == 0 && bin_sums) {
             for (int i = threadIdx.x; i < k.Dd; i += blockDim.x) {
-                const float sum = bins[i];
-                if (sum != 0.0f) {
-                    float *dst = d_depth + (size_t)t * k.Dd + i;
+                float sum = bins[i];
+                float *dst = d_depth + (size_t)t * k.Dd + i;
+                if (persistent) {
+                    if (any_spill) {
+                        float *o = ps.ovf_depth + (size_t)t * k.Dd + i;
+                        sum += *o;
+                        *o = 0.0f;
+                    }
+                    if (fresh) *dst = sum;
+                    else *dst += sum;
+                } else if (sum != 0.0f) {
                     if (shared_texel) atomic_add_f32(dst, sum);
                     else if (store_only) *dst = sum;
                     else *dst += sum;
@@ -274,9 +322,27 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             float sum = 0.0f;
             for (int w = 0; w < nw; ++w) sum += part[w * stride + span + threadIdx.x];
             float *dst = d_depth + (size_t)t * 2 + threadIdx.x;
-            if (shared_texel) atomic_add_f32(dst, sum);
+            if (persistent) {
+                if (any_spill) {
+                    float *o = ps.ovf_depth + (size_t)t * 2 + threadIdx.x;
+                    sum += *o;
+                    *o = 0.0f;
+                }
+                if (fresh) *dst = sum;
+                else *dst += sum;
+            } else if (shared_texel) atomic_add_f32(dst, sum);
             else if (store_only) *dst = sum;
             else *dst += sum;
+        } else if (c0 == 0 && persistent && d_depth != nullptr && !depth_from_pairs) {
+            // the cell pass added the whole depth gradient of this texel to the workspace's buffer
+            for (int i = threadIdx.x; i < k.Dd; i += blockDim.x) {
+                float *o = ps.ovf_depth + (size_t)t * k.Dd + i;
+                const float sum = *o;
+                *o = 0.0f;
+                float *dst = d_depth + (size_t)t * k.Dd + i;
+                if (fresh) *dst = sum;
+                else *dst += sum;
+            }
         }
     }
 }

@@ -242,7 +242,8 @@ int launch_columns(const Plan &pl, const ColParams &cp, size_t lds, const float 
 
 template <typename T, int VEC, int FILL>
 int launch_cells(const Plan &pl, const float *go, const void *depth, const void *feats, const float *proj,
-                 float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap, hipStream_t st) {
+                 float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap, hipStream_t st,
+                 int *epoch = nullptr, int set_stride = 0) {
     dim3 grid(pl.k.n_blocks), block(kWave * pl.k.waves);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
@@ -250,11 +251,11 @@ int launch_cells(const Plan &pl, const float *go, const void *depth, const void 
     prof::Scope timer(FILL ? prof::kBackwardCells : prof::kBackwardScatter, st);
     switch (pl.cpl) {
         case 1: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 1, FILL>, lds)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride); break;
         case 2: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 2, FILL>, lds)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride); break;
         default: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 4, FILL>, lds)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap); break;
+                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride); break;
     }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
@@ -262,17 +263,17 @@ int launch_cells(const Plan &pl, const float *go, const void *depth, const void 
 template <int FILL>
 int dispatch_cells(const fbev_problem *p, const Plan &pl, const float *go, const void *depth, const void *feats,
                    const float *proj, float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap,
-                   hipStream_t st) {
+                   hipStream_t st, int *epoch = nullptr, int set_stride = 0) {
     switch (p->in_dtype) {
         case FBEV_F32:
-            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st)
-                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st);
+            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride)
+                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride);
         case FBEV_F16:
-            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st)
-                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st);
+            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride)
+                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride);
         default:
-            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st)
-                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st);
+            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride)
+                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride);
     }
 }
 
@@ -301,6 +302,26 @@ long long chunk_count(const fbev_problem *p) {
 }
 size_t ws_index_bytes(const fbev_problem *p) {
     return ((size_t)(counter_count(p) + chunk_count(p) + 1) * sizeof(int) + 255) / 256 * 256;
+}
+
+// A persistent workspace (fixed segments only) starts with
+//   [256 bytes: the two call counters][two sets of texels * kFixedReplicas claim counters]
+//   [a depth-gradient and a feature-gradient buffer of the workspace's own], each padded to 256 bytes,
+// then the pairs.  fbev_backward_workspace_init zero-fills all of it but the pairs, once.
+struct PersistLayout {
+    size_t sets, ovf_depth, ovf_feats, pairs;      // byte offsets
+    long long set_stride;                          // ints between the two sets
+};
+PersistLayout persist_layout(const fbev_problem *p) {
+    auto pad = [](size_t n) { return (n + 255) / 256 * 256; };
+    const size_t texels = (size_t)texel_count(p);
+    PersistLayout l;
+    l.set_stride = (long long)texels * kFixedReplicas;
+    l.sets = 256;
+    l.ovf_depth = l.sets + pad(2 * (size_t)l.set_stride * sizeof(int));
+    l.ovf_feats = l.ovf_depth + pad(texels * p->depth_bins * sizeof(float));
+    l.pairs = l.ovf_feats + pad(texels * p->channels * sizeof(float));
+    return l;
 }
 
 int launch_zero(int *a, long long na, float *b, long long nb, float *c, long long nc, hipStream_t st) {
@@ -352,7 +373,7 @@ int scratch_of_current_device(void **out) {
 
 int backward_gather_impl(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
                          const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
-                         size_t workspace_bytes, void *stream) {
+                         size_t workspace_bytes, void *stream, bool persistent = false) {
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
     rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
@@ -360,7 +381,8 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     if (!d_depth && !d_feats) return FBEV_OK;
     if (!workspace) return FBEV_ERR_NULL;
     if ((uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
-    const size_t index_bytes = ws_index_bytes(p);
+    const PersistLayout lay = persist_layout(p);
+    const size_t index_bytes = persistent ? lay.pairs : ws_index_bytes(p);
     if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
     // pair positions are 32-bit: every sample must be countable
     if (sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
@@ -374,8 +396,9 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl, kCellPassWaves);
     if (rc != FBEV_OK) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int *cursor = static_cast<int *>(workspace);
-    Pair *pairs = reinterpret_cast<Pair *>(static_cast<char *>(workspace) + index_bytes);
+    char *base = static_cast<char *>(workspace);
+    int *cursor = persistent ? reinterpret_cast<int *>(base + lay.sets) : static_cast<int *>(workspace);
+    Pair *pairs = reinterpret_cast<Pair *>(base + index_bytes);
     const long long texels = texel_count(p);
     const long long counters = counter_count(p), chunks = chunk_count(p);
     int *chunk_prefix = cursor + counters;
@@ -385,10 +408,25 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     // are not needed.  (A texel that outgrows its segments falls back to atomics, like a full
     // pair array does.)  Smaller workspaces are packed exactly: count, scan, fill.
     const bool fixed = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (texels * kFixedReplicas) >= kFixedMinSegment;
+    if (persistent && !fixed) return FBEV_ERR_SHAPE;      // a persistent workspace holds the worst case
     const int seg_cap = fixed ? (int)(cap / (texels * kFixedReplicas)) : 0;
-    rc = launch_zero(cursor, fixed ? texels * kFixedReplicas : counters, accumulate ? nullptr : d_depth,
-                     texels * p->depth_bins, accumulate ? nullptr : d_feats, texels * p->channels, st);
-    if (rc != FBEV_OK) return rc;
+    // what the two kernels get when the workspace is persistent: no zero-fill launch then
+    Persist ps = {nullptr, nullptr, 0, nullptr, nullptr};
+    float *cells_dd = d_depth, *cells_df = d_feats;
+    if (persistent) {
+        ps.epoch = reinterpret_cast<int *>(base);
+        ps.sets = cursor;
+        ps.set_stride = (int)lay.set_stride;
+        ps.ovf_depth = reinterpret_cast<float *>(base + lay.ovf_depth);
+        ps.ovf_feats = reinterpret_cast<float *>(base + lay.ovf_feats);
+        // the cell pass adds what it cannot file to the workspace's own gradient buffers
+        if (d_depth) cells_dd = ps.ovf_depth;
+        if (d_feats) cells_df = ps.ovf_feats;
+    } else {
+        rc = launch_zero(cursor, fixed ? texels * kFixedReplicas : counters, accumulate ? nullptr : d_depth,
+                         texels * p->depth_bins, accumulate ? nullptr : d_feats, texels * p->channels, st);
+        if (rc != FBEV_OK) return rc;
+    }
     if (!fixed) {
         switch (p->in_dtype) {
             case FBEV_F32: rc = launch_count<float>(pl, depth, proj, cursor, st); break;
@@ -412,10 +450,10 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     const int cap_arg = fixed ? seg_cap : cap;
     // samples a claim counter gets if every sample is kept
     const bool claim_runs = sample_count(p) / (fixed ? texels * kFixedReplicas : counters) >= kClaimRunsFrom;
-    rc = claim_runs ? dispatch_cells<2>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
-                                        cap_arg, st)
-                    : dispatch_cells<1>(p, pl, grad_out, depth, feats, proj, d_depth, d_feats, prefix_arg, cursor, pairs,
-                                        cap_arg, st);
+    rc = claim_runs ? dispatch_cells<2>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs,
+                                        cap_arg, st, ps.epoch, ps.set_stride)
+                    : dispatch_cells<1>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs,
+                                        cap_arg, st, ps.epoch, ps.set_stride);
     if (rc != FBEV_OK) return rc;
 
     // texel pass: rows of grad_out are fp32, so 128-bit gathers need C % 4 == 0 and aligned rows
@@ -440,13 +478,15 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
         (d_depth != nullptr && pl.k.C <= pl.k.lanes_per_slot * pl.vec * pl.cpl && pl.k.bin_bits >= 0) ? 1 : 0;
     const size_t lds = ((size_t)texel_waves * kWave * 2 + (size_t)nw * (lpr * vec + 2) +
                         (p->depth_distribution == FBEV_CATEGORICAL ? p->depth_bins : 0)) * sizeof(float);
-    long long want_split = kTexelSplitBelow / texels;
+    // (the blocks of a split texel add their shares with atomics, which needs cleared buffers: a
+    // persistent workspace, whose calls clear nothing, keeps one block per texel)
+    long long want_split = persistent ? 1 : kTexelSplitBelow / texels;
     const unsigned n_split = (unsigned)(want_split < 1 ? 1 : (want_split > kTexelMaxSplit ? kTexelMaxSplit : want_split));
     prof::Scope timer(prof::kBackwardTexel, st);
     const dim3 tgrid((unsigned)texels, n_split), tblock(kWave * texel_waves);
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats,
-                           lpr, from_pairs, accumulate ? 0 : 1);
+                           lpr, from_pairs, accumulate ? 0 : 1, ps);
     };
     if (vec4) {
         if (texel_waves == 1) launch(fbev_backward_texel_kernel<4, 1>);
@@ -458,6 +498,17 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
         else launch(fbev_backward_texel_kernel<1, kWavesPerBlock>);
     }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+// Zero-fill everything of a persistent workspace but its pairs.
+int workspace_init_impl(const fbev_problem *p, void *workspace, size_t workspace_bytes, hipStream_t st) {
+    int rc = validate(p, true);
+    if (rc != FBEV_OK) return rc;
+    if (!workspace) return FBEV_ERR_NULL;
+    if ((uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
+    const PersistLayout lay = persist_layout(p);
+    if (workspace_bytes < lay.pairs) return FBEV_ERR_SHAPE;
+    return launch_zero(static_cast<int *>(workspace), (long long)(lay.pairs / sizeof(int)), nullptr, 0, nullptr, 0, st);
 }
 
 }  // namespace
@@ -571,6 +622,25 @@ int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const voi
                          size_t workspace_bytes, void *stream) {
     return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
                                 workspace_bytes, stream);
+}
+
+size_t fbev_backward_persistent_workspace_bytes(const fbev_problem *p) {
+    if (validate(p, true) != FBEV_OK) return 0;
+    // room for every sample, and never less than the shortest segment the fixed layout works with
+    const uint64_t least = (uint64_t)texel_count(p) * kFixedReplicas * kFixedMinSegment;
+    const uint64_t pairs = fbev_backward_max_pairs(p) > least ? fbev_backward_max_pairs(p) : least;
+    return persist_layout(p).pairs + (size_t)pairs * sizeof(Pair);
+}
+
+int fbev_backward_workspace_init(const fbev_problem *p, void *workspace, size_t workspace_bytes, void *stream) {
+    return workspace_init_impl(p, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int fbev_backward_gather_persistent(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                                    const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+    return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
+                                workspace_bytes, stream, true);
 }
 
 int fbev_backward_gather_static(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,

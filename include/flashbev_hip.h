@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 6
+#define FBEV_ABI_VERSION 7
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -129,6 +129,29 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
 int fbev_backward_gather(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
                          const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
                          size_t workspace_bytes, void *stream);
+
+/*
+ * fbev_backward_gather on a workspace that persists between calls: two launches (cell pass, texel
+ * pass) instead of three, because nothing has to be cleared at the start of a call.  The workspace
+ * holds two sets of claim counters (a call claims in one, its texel pass clears the other for the
+ * next call; a call counter kept in the workspace selects the set, so a call captured into a HIP
+ * graph can be replayed) and gradient buffers of its own for what the cell pass cannot file under
+ * a texel (a full segment), which the texel pass takes over and clears again.  Every element of
+ * d_depth and d_feats is stored (accumulate == 0) or added to (accumulate != 0) by the texel pass.
+ * Contract: `workspace` has at least fbev_backward_persistent_workspace_bytes(p) bytes (room for
+ * every sample: fixed segments), is 16-byte aligned, was prepared by fbev_backward_workspace_init
+ * for the same p once (again whenever batch, cameras, feature-map size, channels or depth bins
+ * change, or after anything else wrote to it), and is used by one call at a time (calls on one
+ * stream are ordered; calls that overlap in time race).  A call that fails, or is not followed by
+ * its own completion, leaves the workspace undefined: prepare it again.  Same results as
+ * fbev_backward_gather.  No counterpart in the reference, whose backward allocates nothing and
+ * scatters with atomics (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:867-937).
+ */
+size_t fbev_backward_persistent_workspace_bytes(const fbev_problem *p);
+int fbev_backward_workspace_init(const fbev_problem *p, void *workspace, size_t workspace_bytes, void *stream);
+int fbev_backward_gather_persistent(const fbev_problem *p, const float *grad_out, const void *depth,
+                                    const void *feats, const float *proj, float *d_depth, float *d_feats,
+                                    int accumulate, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * fbev_backward_gather without a workspace argument and without any allocation: the inverse map

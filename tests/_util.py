@@ -81,11 +81,13 @@ def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEA
     """Backward through the C ABI.  mode "scatter" = fbev_backward, "gather" = fbev_backward_gather
     with a workspace for `pair_capacity` pairs (default: the worst case, which selects fixed
     per-texel segments; "gather_counted" defaults to half of that, the exactly packed layout), "columns" =
-    fbev_backward_columns overwriting NaN-filled buffers with recounted cell counts,
+    fbev_backward_columns overwriting NaN-filled buffers with recounted cell counts, "persistent" =
+    fbev_backward_gather_persistent on a workspace prepared once (three calls in a row, the last one returned),
     "columns_acc" = the same accumulating into zero-filled buffers with the forward's counts."""
     p = problem_for(x, w, dist, thr, eps, reduction)
     dev = x["image_feats"].device
-    overwrite = mode in ("columns", "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite")
+    overwrite = mode in ("columns", "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite",
+                         "persistent_overwrite")
     fill = float("nan") if overwrite else 0.0
     dd = torch.full(x["depth_params"].shape, fill, dtype=torch.float32, device=dev) if want[0] else None
     df = torch.full(x["image_feats"].shape, fill, dtype=torch.float32, device=dev) if want[1] else None
@@ -108,6 +110,21 @@ def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEA
             _, cnt = capi_forward(x, w, dist, thr, eps, reduction, with_count=True)
             capi.check(capi.backward_columns(p, *args, cnt.data_ptr(), ddp, dfp, True, None, 0, st),
                        "fbev_backward_columns")
+    elif mode in ("persistent", "persistent_overwrite"):
+        # a workspace prepared once, then three calls in a row on it (the claim-counter sets alternate);
+        # the last call's gradients are returned
+        nbytes = capi.backward_persistent_workspace_bytes(p)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(0x5A)
+        capi.check(capi.backward_workspace_init(p, ws.data_ptr(), nbytes, st), "fbev_backward_workspace_init")
+        for call in range(3):
+            if dd is not None:
+                dd.fill_(fill)
+            if df is not None:
+                df.fill_(fill)
+            capi.check(capi.backward_gather_persistent(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
+                                                       x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(),
+                                                       ddp, dfp, ws.data_ptr(), nbytes, st, accumulate=not overwrite),
+                       "fbev_backward_gather_persistent")
     else:
         cap = pair_capacity
         if cap is None:

@@ -306,3 +306,40 @@ def test_operator_backward_variants_agree(monkeypatch, env):
         monkeypatch.setenv(key, value)
     got_f, got_d = grads()
     assert torch.allclose(got_f, want_f, rtol=1e-4, atol=1e-5) and torch.allclose(got_d, want_d, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("extra", [["--num-height-bins", "4", "8"], ["--num-cameras-list", "1", "6", "--module"]])
+def test_latency_sweep_harness_runs_and_keeps_the_reference_record_layout(extra, tmp_path):
+    """profile_latency.run on a two-point sweep (a small grid, few timed calls): one record per point
+    with the keys of the reference's record (tools/profile_latency.py:176-183: method, num_height_bins,
+    num_cameras, z_resolution, depth_weight_threshold, the method's configuration, the statistics of
+    tools/utils/benchmark_utils.py:71-92) and the file layout of tools/profile_latency.py:405-430."""
+    import json
+
+    from flashbev_amd import profile_latency as pl
+
+    out_json = str(tmp_path / "sweep.json")
+    args = pl.parse_args(extra + ["--grid-x", "-20", "20", "1", "--grid-y", "-20", "20", "1", "--num-warmup", "2",
+                                  "--num-iterations", "5", "--in-channels", "32", "--out-channels", "16",
+                                  "--output-json", out_json])
+    pl.main(extra + ["--grid-x", "-20", "20", "1", "--grid-y", "-20", "20", "1", "--num-warmup", "2",
+                     "--num-iterations", "5", "--in-channels", "32", "--out-channels", "16", "--output-json", out_json])
+    out = json.load(open(out_json))
+    exp = pl.experiment_of(args)
+    assert set(out) == {"config", "results"}
+    assert set(out["config"]) == {"batch_size", "num_cameras", "feature_h", "feature_w", "in_channels", "out_channels",
+                                  "input_h", "input_w", "downsample", "num_warmup", "num_iterations", "device",
+                                  "grid_config", "num_height_bins", "num_cameras_list", "depth_weight_threshold_list",
+                                  "z_resolutions", "experiment_type"}
+    assert out["config"]["experiment_type"] == exp["experiment_type"]
+    assert len(out["results"]) == 2
+    reference_keys = {"method", "num_height_bins", "num_cameras", "z_resolution", "depth_weight_threshold",
+                      "fuse_projection", "use_bev_pool", "latency_mean_ms", "latency_std_ms", "latency_min_ms",
+                      "latency_max_ms", "latency_p50_ms", "latency_p95_ms", "latency_p99_ms",
+                      "peak_memory_allocated_mb", "peak_memory_reserved_mb"}
+    for rec, value in zip(out["results"], exp["values"]):
+        assert reference_keys <= set(rec), reference_keys - set(rec)
+        assert rec["method"] == "FlashBEV(ours)" and rec["fuse_projection"] is True
+        assert rec["num_height_bins" if exp["experiment_type"] == "height_bins" else "num_cameras"] == value
+        assert 0.0 < rec["latency_min_ms"] <= rec["latency_p50_ms"] <= rec["latency_max_ms"] < 1000.0

@@ -57,7 +57,8 @@ def test_forward_matches_c_oracle(name, dist, thr):
 @pytest.mark.parametrize("name", ["cfg1_tiny", "cfg2_surround"])
 @pytest.mark.parametrize("dist", [0, 1, 2])
 @pytest.mark.parametrize("mode", ["scatter", "gather", "gather_counted", "columns", "columns_acc",
-                                  "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite"])
+                                  "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite",
+                                  "persistent", "persistent_overwrite"])
 def test_backward_matches_c_oracle(name, dist, mode):
     w, x = _inputs(name, dist)
     dd, df = U.capi_backward(x, w, dist, mode=mode)

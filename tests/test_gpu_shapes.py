@@ -22,7 +22,7 @@ def small(name="cfg2_surround", **kw):
     return dataclasses.replace(WORKLOADS[name], **kw)
 
 
-def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "gather_counted", "columns"), fwd_tol=(1e-4, 1e-5),
+def check_all(w, x, dist, thr=1e-6, modes=("scatter", "gather", "gather_counted", "columns", "persistent_overwrite"), fwd_tol=(1e-4, 1e-5),
               bwd_tol=(1e-4, 1e-5)):
     out = U.capi_forward(x, w, dist, thr).cpu().numpy()
     want = U.oracle_forward(x, w, dist, thr)
@@ -269,7 +269,8 @@ def test_fixed_segments_overflow_falls_back_to_atomics(dist):
     assert seg_cap >= 16 and per_texel.max() > 8 * seg_cap, (seg_cap, per_texel.max())
     # a gradient element here is a sum of thousands of fp32 terms whose order the overflow atomics do not
     # fix: three times the usual tolerance (observed: up to 1.01 times the usual one)
-    check_all(w, x, dist, thr=0.0, modes=("gather", "gather_overwrite", "gather_counted"), bwd_tol=(3e-4, 3e-5))
+    check_all(w, x, dist, thr=0.0, modes=("gather", "gather_overwrite", "gather_counted", "persistent",
+                                          "persistent_overwrite"), bwd_tol=(3e-4, 3e-5))
 
 
 def test_the_reference_calibration_fixture():
@@ -360,7 +361,8 @@ def test_tiny_feature_maps_and_clamped_corners(feat_hw, dist):
         idx = geo["idx"][valid]
         assert (idx[:, 0] == idx[:, 1]).any() or feat_hw == (16, 44)      # some u1 clamped onto u0
     print(f"[case] feat_hw={feat_hw} dist={dist} valid={int(valid.sum())}", flush=True)
-    check_all(w, x, dist, thr=0.0, modes=("scatter", "gather", "gather_overwrite", "gather_counted", "columns"))
+    check_all(w, x, dist, thr=0.0, modes=("scatter", "gather", "gather_overwrite", "gather_counted", "columns", "persistent",
+                                          "persistent_overwrite"))
 
 
 @pytest.mark.parametrize("feat_hw", [(4, 6), (1, 2)])
@@ -376,7 +378,7 @@ def test_many_samples_per_claim_counter_claim_by_runs(feat_hw, dist):
     x = make_inputs(w, MODEL[dist], device="cuda", with_grad_out=True)
     for thr in (0.0, 1e-6):
         print(f"[case] claim runs feat_hw={feat_hw} dist={dist} thr={thr}", flush=True)
-        check_all(w, x, dist, thr=thr, modes=("gather", "gather_overwrite", "gather_counted"))
+        check_all(w, x, dist, thr=thr, modes=("gather", "gather_overwrite", "gather_counted", "persistent_overwrite"))
 
 
 @pytest.mark.parametrize("channels,gz,dtype", [(80, 50, torch.float32), (64, 40, torch.float32),
