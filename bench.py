@@ -4,19 +4,23 @@
 
 One step = one forward plus one backward pass of the operator over one batch of seeded
 synthetic input that is already resident in HBM: the forward kernel (which also records the
-per-cell sample counts) and the backward kernels (whose first launch zero-fills the two
-gradient buffers), all queued on PyTorch's current stream through the extension module.  The default workload is the 6-camera 128x128x8 fp32 configuration
+per-cell sample counts) and the two backward kernels of the inverse map on a workspace that was
+prepared once, before the timed region (cell pass, texel pass; every gradient element is stored by
+the texel pass), all queued on PyTorch's current stream through the extension module.  The default workload is the 6-camera 128x128x8 fp32 configuration
 (``cfg2_surround``) with the reference benchmark's depth model (per-pixel Laplace
 parameters, tools/config/config.yaml:29).  The single JSON line printed on stdout carries
   value / ms_per_step   forward+backward latency per step (ms), K eagerly queued steps between two
                         synchronisations; ms_per_step_graph is the same step captured into a HIP
                         graph and replayed K times (checked against the eager result first) --
                         on this machine the eager queue is already GPU-bound and no slower
-  roofline              the dominant pass (the backward, five kernel launches): its compulsory
+  roofline              the dominant pass (the backward: cell pass + texel pass): its compulsory
                         bytes / the summed mean durations of its kernels, measured with HIP
                         events the library records around every one of its launches over a
                         second run of the same K steps, against the 8 TB/s HBM3E peak;
                         "kernels" lists every kernel's mean duration and launch count
+  other_workloads       the high-resolution inference and the training-size configurations timed in the
+                        same run (forward; forward and backward), with their compulsory bytes and
+                        fraction of the HBM peak: the sizes at which that fraction means something
   cpu_baseline          the dense PyTorch restatement of the reference's pooling path
                         (oracle/dense_torch.py), forward+backward via autograd on the host
                         cores, same workload -- a reported baseline, not a target.
@@ -44,19 +48,26 @@ from flashbev_amd.workloads import WORKLOADS, algorithmic_bytes, make_inputs  # 
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
-# counters read for a 256 MiB copy (x2.000 / x1.000); see profiles/.  Only for the workload
-# and kernels the counters were collected on; anything else reports null.
-MEASURED_TRAFFIC = {
-    ("cfg2_surround", "laplace", 0): {"backward": 22.4e6, "forward": 8.40e6,
-                                      "source": "profiles/cfg2_surround_laplace_fwd_bwd_gather.md"},
-}
+# counters read for a 256 MiB copy: kept beside the profile summaries they come from, keyed
+# "workload/depth model/backward mode".  Anything the counters were not collected on reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(workload: str, depth: str, backward_mode: int):
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            return json.load(fh).get(f"{workload}/{depth}/{backward_mode}")
+    except (OSError, ValueError):
+        return None
+
+
 DIST_OF = {"gaussian": (0, "parametric"), "laplace": (1, "parametric"), "categorical": (2, "categorical")}
 
 
 class Runner:
     """Pre-allocated buffers and the four queued operations of one step."""
 
-    def __init__(self, w, depth_name: str, device: str = "cuda:0", backward_mode: int = 0):
+    def __init__(self, w, depth_name: str, device: str = "cuda:0", backward_mode: int = 0, persistent: bool = True):
         self.w = w
         self.backward_mode = backward_mode
         self.dist, self.model = DIST_OF[depth_name]
@@ -71,6 +82,16 @@ class Runner:
         self.counts = torch.empty((B, gy, gx), dtype=torch.float32, device=device)
         self.vmin, self.vsize = voxel_geometry(w.roi_range, w.grid_size)
         self.eps, self.thr = 1e-6, 1e-6
+        # the inverse map's workspace, prepared once (what the autograd operator keeps per shape);
+        # persistent=False takes a fresh workspace from the caching allocator in every call instead
+        self.workspace = None
+        if persistent and backward_mode in (0, 2):
+            nbytes = self.ext.backward_workspace_bytes(x["depth_params"], x["image_feats"], x["projection_matrices"],
+                                                       x["feature_size"], x["image_size"], x["grid_size"], self.dist)
+            if nbytes:
+                self.workspace = self.ext.prepare_backward_workspace(
+                    x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
+                    x["image_size"], x["grid_size"], self.dist)
 
     def forward(self):
         x, w = self.x, self.w
@@ -86,7 +107,7 @@ class Runner:
             x["grad_out"], x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
             x["image_size"], x["roi_range"], x["grid_size"], self.d_depth, self.d_feats, self.out.numel(),
             self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0, self.backward_mode, -1,
-            self.counts, False)
+            self.counts, False, self.workspace)
 
 
 def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
@@ -181,14 +202,19 @@ def time_operator_steps(r: Runner, steps: int, warmup: int):
             else:
                 feats.grad = depth.grad = None
                 flash_bevpool(image_feats=feats, depth_params=depth, **kw).backward(x["grad_out"])
-        for _ in range(warmup):
+        for _ in range(max(warmup, 10)):
             step()
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            step()
-        torch.cuda.synchronize()
-        got[name] = (time.perf_counter() - t0) * 1e3 / steps
+        # five chunks, the median reported: a one-off stall of the allocator or the host (tens of
+        # milliseconds, seen once per process) would otherwise own a short run
+        chunks = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(max(1, steps // 5)):
+                step()
+            torch.cuda.synchronize()
+            chunks.append((time.perf_counter() - t0) * 1e3 / max(1, steps // 5))
+        got[name] = statistics.median(chunks)
     return got
 
 
@@ -228,6 +254,34 @@ def cpu_baseline(w, depth_name: str, budget_s: float = 20.0, max_runs: int = 5):
             break
     return {"value": statistics.mean(times) * 1e3, "unit": "ms", "cores": cores, "kind": "port",
             "sample": f"{w.name} full workload, dense PyTorch path fwd+bwd, 1 warm-up + {len(times)} timed runs"}
+
+
+def other_workloads(steps: int, warmup: int, backward_mode: int):
+    """The two large configurations in the same run: high-resolution inference (bf16, forward) and
+    training size (fp16, forward and backward), Laplace depth; event-timed calls, compulsory bytes
+    (every operand tensor once) and the fraction of the HBM peak they amount to."""
+    got = {}
+    for name, with_backward in (("cfg4_hires", False), ("cfg5_train", True)):
+        w = WORKLOADS[name]
+        r = Runner(w, "laplace", backward_mode=backward_mode)
+        ms, fwd, bwd = time_steps(r, steps, warmup, with_backward)
+        fb, bb = algorithmic_bytes(w, r.model, False), algorithmic_bytes(w, r.model, True)
+        f_ms = statistics.mean(fwd)
+        rec = {"dtype": str(w.dtype).replace("torch.", ""), "depth_model": "laplace", "steps": steps,
+               "batch": w.batch, "channels": w.channels, "feat_hw": list(w.feat_hw), "grid": list(w.grid_size),
+               "forward": {"ms": f_ms, "algorithmic_bytes": fb, "GBps": fb / f_ms / 1e6,
+                           "frac_hbm": fb / f_ms / 1e6 / HBM_PEAK_GBS}}
+        if with_backward:
+            b_ms = statistics.mean(bwd)
+            rec["backward"] = {"ms": b_ms, "algorithmic_bytes": bb, "GBps": bb / b_ms / 1e6,
+                               "frac_hbm": bb / b_ms / 1e6 / HBM_PEAK_GBS}
+            rec["ms_per_step_fwd_bwd"] = ms
+            rec["frac_hbm_fwd_bwd"] = (fb + bb) / ms / 1e6 / HBM_PEAK_GBS
+        rec["kept_samples"] = int(r.counts.sum().item())
+        got[name] = rec
+        del r
+        torch.cuda.empty_cache()
+    return got
 
 
 def stats(v):
@@ -285,6 +339,8 @@ def main():
     ap.add_argument("--table", action="store_true")
     ap.add_argument("--table-dir", default="bench_out", help="directory (under the repository) for the --table files")
     ap.add_argument("--no-graph", action="store_true", help="time eagerly queued steps only")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the two large configurations otherwise timed beside the default workload")
     ap.add_argument("--backward-mode", type=int, default=0, choices=(0, 1, 2, 3),
                     help="0 auto (default), 1 atomic scatter, 2 inverse-map gather, 3 column owner")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
@@ -313,6 +369,11 @@ def main():
     eager_ms, fwd, bwd = time_steps(r, args.steps, args.warmup, True)
     graph_ms = None if args.no_graph else time_graph_steps(r, args.steps, args.warmup)
     ms = eager_ms
+    # the same step with a per-call workspace (three backward launches: the first clears the claim
+    # counters and the gradient buffers), what a caller without a persistent workspace gets
+    r0 = Runner(w, args.depth, backward_mode=args.backward_mode, persistent=False)
+    percall_ms = time_steps(r0, args.steps, args.warmup, True)[0]
+    del r0
     kernels = profile_steps(r, args.steps)
     op_ms = time_operator_steps(r, args.steps, args.warmup)
     fwd_ms, bwd_ms = statistics.mean(fwd), statistics.mean(bwd)
@@ -327,7 +388,7 @@ def main():
     k_ms, k_bytes, k_names = (bwd_k_ms, bb, bwd_names) if dominant == "backward" else (fwd_k_ms, fb, fwd_names)
     achieved = k_bytes / k_ms / 1e6  # GB/s
     top = max(kernels, key=lambda k: kernels[k]["mean_us"] * kernels[k]["calls_per_step"])
-    traffic = MEASURED_TRAFFIC.get((w.name, args.depth, args.backward_mode))
+    traffic = measured_traffic(w.name, args.depth, args.backward_mode)
     line = {
         "metric": "BEV-pool fwd+bwd latency (ms) & effective HBM GB/s, 6 cams 128x128xZ=8, 1 GPU",
         "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -337,9 +398,9 @@ def main():
         "config": {"workload": w.name, "depth_model": args.depth, "batch": w.batch, "cams": w.num_cams,
                    "channels": w.channels, "feat_hw": list(w.feat_hw), "grid": list(w.grid_size),
                    "backward": {0: "auto", 1: "atomic scatter", 2: "inverse-map gather", 3: "column owner"}[args.backward_mode],
-                   "step": "forward kernel + backward kernels (gradient zero-fill folded into the first)",
+                   "step": "forward kernel + cell pass + texel pass (inverse map on a workspace prepared once)",
                    "submission": "eager launches on one stream"},
-        "ms_per_step_eager": eager_ms, "ms_per_step_graph": graph_ms,
+        "ms_per_step_eager": eager_ms, "ms_per_step_graph": graph_ms, "ms_per_step_per_call_workspace": percall_ms,
         "fwd_call_ms": stats(fwd), "bwd_call_ms": stats(bwd),
         # the same work through the autograd operator, output and gradient allocation included
         "operator_ms_incl_alloc": {"fwd": op_ms["fwd"], "fwd_bwd": op_ms["fwd_bwd"]},
@@ -373,6 +434,8 @@ def main():
                         "kept_samples": int(r2.counts.sum().item())}
         del r2
     line["other_depth_models"] = others
+    if args.workload == "cfg2_surround" and not args.no_other_workloads:
+        line["other_workloads"] = other_workloads(max(10, args.steps // 10), max(3, args.warmup // 4), args.backward_mode)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, args.depth)
     if args.table:

@@ -44,12 +44,27 @@ int dtype_code(const at::Tensor &t, const char *name) {
 // costs one synchronous copy, as in the reference (flash_bevpool.cpp:118-124).
 std::vector<int64_t> host_ints(const at::Tensor &t, int64_t n, const char *name) {
     TORCH_CHECK(t.numel() == n, "flashbevpool_ext: ", name, " must have ", n, " elements, got ", t.numel());
+    // host tensors in their usual types are read in place (no temporary tensor per call)
+    if (t.device().is_cpu() && t.is_contiguous()) {
+        if (t.scalar_type() == at::kInt) {
+            const int32_t *v = t.data_ptr<int32_t>();
+            return std::vector<int64_t>(v, v + n);
+        }
+        if (t.scalar_type() == at::kLong) {
+            const int64_t *v = t.data_ptr<int64_t>();
+            return std::vector<int64_t>(v, v + n);
+        }
+    }
     at::Tensor h = t.to(at::kCPU, at::kLong).contiguous();
     return std::vector<int64_t>(h.data_ptr<int64_t>(), h.data_ptr<int64_t>() + n);
 }
 
 std::vector<float> host_floats(const at::Tensor &t, int64_t n, const char *name) {
     TORCH_CHECK(t.numel() == n, "flashbevpool_ext: ", name, " must have ", n, " elements, got ", t.numel());
+    if (t.device().is_cpu() && t.is_contiguous() && t.scalar_type() == at::kFloat) {
+        const float *v = t.data_ptr<float>();
+        return std::vector<float>(v, v + n);
+    }
     at::Tensor h = t.to(at::kCPU, at::kFloat).contiguous();
     return std::vector<float>(h.data_ptr<float>(), h.data_ptr<float>() + n);
 }
@@ -184,7 +199,8 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                             std::optional<at::Tensor> depth_params_grad, std::optional<at::Tensor> image_feats_grad,
                             int64_t total_threads, int depth_distribution, float epsilon, float depth_weight_threshold,
                             float depth_min, float depth_step, int reduction, int backward_mode,
-                            int64_t pair_capacity, std::optional<at::Tensor> cell_count, bool accumulate) {
+                            int64_t pair_capacity, std::optional<at::Tensor> cell_count, bool accumulate,
+                            std::optional<at::Tensor> workspace) {
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
     auto roi = host_floats(roi_range, 6, "roi_range");
@@ -255,7 +271,17 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                                     projection_matrices.data_ptr<float>(), dd, df, accumulate ? 1 : 0, ws.data_ptr(),
                                     bytes, st);
     };
-    if (backward_mode == 1) {
+    if (workspace.has_value() && workspace->defined()) {
+        // a workspace from prepare_backward_workspace: the inverse map in two launches, nothing allocated
+        TORCH_CHECK(backward_mode == 0 || backward_mode == 2,
+                    "flashbevpool_ext: a persistent workspace goes with backward_mode 0 (auto) or 2 (gather)");
+        check_dev(*workspace, depth_params, "workspace");
+        TORCH_CHECK(workspace->scalar_type() == at::kByte, "flashbevpool_ext: workspace must be a uint8 tensor");
+        raise_on(fbev_backward_gather_persistent(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(),
+                                                 image_feats.data_ptr(), projection_matrices.data_ptr<float>(), dd, df,
+                                                 accumulate ? 1 : 0, workspace->data_ptr(), (size_t)workspace->numel(), st),
+                 "fbev_backward_gather_persistent");
+    } else if (backward_mode == 1) {
         raise_on(fbev_backward(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
                                projection_matrices.data_ptr<float>(), dd, df, accumulate ? 1 : 0, st),
                  "fbev_backward");
@@ -269,6 +295,34 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
         if (rc == FBEV_ERR_TOO_LARGE) raise_on(run_columns(), "fbev_backward_columns");
         else raise_on(rc, "fbev_backward_gather");
     }
+}
+
+// Bytes of a persistent inverse-map workspace for these tensors (0: the problem is beyond the
+// inverse map's 32-bit positions), and a workspace allocated and prepared on the current stream.
+int64_t backward_workspace_bytes(const at::Tensor &depth_params, const at::Tensor &image_feats,
+                                 const at::Tensor &projection_matrices, const at::Tensor &feature_size,
+                                 const at::Tensor &image_size, const at::Tensor &grid_size, int depth_distribution) {
+    fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              depth_distribution, 1e-6f, 0.0f, 1.0f, 1.0f, 0);
+    const uint64_t max_pairs = fbev_backward_max_pairs(&p);
+    const uint64_t texels = (uint64_t)p.batch * p.num_cams * p.feat_h * p.feat_w;
+    if (max_pairs == 0 || max_pairs >= (1ull << 31) || texels * 32 >= (1ull << 31)) return 0;
+    return (int64_t)fbev_backward_persistent_workspace_bytes(&p);
+}
+
+at::Tensor prepare_backward_workspace(const at::Tensor &depth_params, const at::Tensor &image_feats,
+                                      const at::Tensor &projection_matrices, const at::Tensor &feature_size,
+                                      const at::Tensor &image_size, const at::Tensor &grid_size,
+                                      int depth_distribution) {
+    fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              depth_distribution, 1e-6f, 0.0f, 1.0f, 1.0f, 0);
+    const size_t bytes = fbev_backward_persistent_workspace_bytes(&p);
+    TORCH_CHECK(bytes > 0, "flashbevpool_ext: no persistent workspace for this problem");
+    at::Tensor ws = at::empty({(int64_t)bytes}, at::TensorOptions().device(depth_params.device()).dtype(at::kByte));
+    DeviceScope scope(depth_params.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
+    raise_on(fbev_backward_workspace_init(&p, ws.data_ptr(), bytes, st), "fbev_backward_workspace_init");
+    return ws;
 }
 
 // Parity hook: per-sample validity mask and bilinear corner indices, [B,gy,gx,N,gz(,4|2)].
@@ -396,7 +450,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("depth_distribution"), py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f,
           py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0,
           py::arg("backward_mode") = 0, py::arg("pair_capacity") = -1, py::arg("cell_count") = py::none(),
-          py::arg("accumulate") = true);
+          py::arg("accumulate") = true, py::arg("workspace") = py::none());
+    m.def("backward_workspace_bytes", &backward_workspace_bytes,
+          "bytes of a persistent inverse-map workspace (0 when the problem is beyond the inverse map)");
+    m.def("prepare_backward_workspace", &prepare_backward_workspace,
+          "a persistent inverse-map workspace, allocated and prepared on the current stream");
     m.def("sample_geometry", &sample_geometry, "per-sample validity mask and corner indices (parity hook)",
           py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
           py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);

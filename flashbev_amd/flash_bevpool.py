@@ -23,6 +23,7 @@ results in the reference either.
 """
 from __future__ import annotations
 
+import collections
 import functools
 import os
 import weakref
@@ -48,7 +49,7 @@ def _backward_mode() -> int:
 
 
 def _pair_capacity(batch: int, cams: int, grid) -> int:
-    """Pair slots of the inverse-map workspace.  Room for every sample (32 bytes each) lets the
+    """Pair slots of a per-call inverse-map workspace.  Room for every sample (32 bytes each) lets the
     library skip its counting passes; FLASHBEV_WORKSPACE_MB (default 16384) bounds the
     allocation, and a smaller workspace is packed exactly instead (-1 = the extension's default,
     room for everything)."""
@@ -57,6 +58,41 @@ def _pair_capacity(batch: int, cams: int, grid) -> int:
     if max_pairs * 32 <= limit_mb * 2 ** 20:
         return -1
     return max(0, int(limit_mb * 2 ** 20) // 32)
+
+
+# Persistent inverse-map workspaces, one per (device, stream, problem shape, depth model): prepared
+# once, then every backward of that shape on that stream is two launches and allocates nothing.  The
+# few most recently used are kept (FLASHBEV_WORKSPACES, default 4; 0 switches them off and every
+# call takes its workspace from the caching allocator instead).
+_workspaces: "collections.OrderedDict" = collections.OrderedDict()
+
+
+def _stream_id(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _persistent_workspace(ext, depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
+                          depth_distribution):
+    keep = int(os.environ.get("FLASHBEV_WORKSPACES", "4"))
+    if keep <= 0:
+        return None, None
+    key = (image_feats.device.index, _stream_id(image_feats.device),
+           tuple(image_feats.shape), depth_params.shape[-1], tuple(grid_t.tolist()), int(depth_distribution))
+    ws = _workspaces.get(key)
+    if ws is None:
+        nbytes = ext.backward_workspace_bytes(depth_params, image_feats, projection_matrices, fs_host, image_t,
+                                              grid_t, int(depth_distribution))
+        limit_mb = float(os.environ.get("FLASHBEV_WORKSPACE_MB", "16384"))
+        if nbytes == 0 or nbytes > limit_mb * 2 ** 20:
+            return None, None
+        ws = ext.prepare_backward_workspace(depth_params, image_feats, projection_matrices, fs_host, image_t,
+                                            grid_t, int(depth_distribution))
+        _workspaces[key] = ws
+        while len(_workspaces) > keep:
+            _workspaces.popitem(last=False)
+    else:
+        _workspaces.move_to_end(key)
+    return key, ws
 
 
 # id(tensor) -> (weak reference, version, values).  Keyed by identity: a mapping keyed by the
@@ -219,11 +255,20 @@ class FlashBEVPool(torch.autograd.Function):
         image_feats_grad = alloc(image_feats.shape, dtype=torch.float32,
                                  device=image_feats.device) if need_feats else None
         if need_depth or need_feats:
-            ext.flash_bevpool_backward(
-                out_grad.contiguous().float(), depth_params, image_feats, projection_matrices,
-                fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
-                ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
-                ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, ctx.pair_capacity, ctx.counts, False)
+            key = ws = None
+            if mode in (0, 2) and ctx.pair_capacity < 0:
+                key, ws = _persistent_workspace(ext, depth_params, image_feats, projection_matrices, fs_host,
+                                                image_t, grid_t, ctx.depth_distribution)
+            try:
+                ext.flash_bevpool_backward(
+                    out_grad.contiguous().float(), depth_params, image_feats, projection_matrices,
+                    fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
+                    ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
+                    ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, ctx.pair_capacity, ctx.counts, False,
+                    ws)
+            except Exception:
+                _workspaces.pop(key, None)       # a failed call leaves a persistent workspace undefined
+                raise
         return (depth_params_grad, image_feats_grad) + (None,) * 14
 
 

@@ -169,11 +169,20 @@ class FakeExt:
         if a[9] is not None:
             a[9].fill_(3.0)
 
+    def backward_workspace_bytes(self, *a):
+        return 4096
+
+    def prepare_backward_workspace(self, *a):
+        self.prepared = getattr(self, "prepared", 0) + 1
+        return torch.zeros(4096, dtype=torch.uint8)
+
 
 @pytest.fixture
 def fake_ext(monkeypatch):
     ext = FakeExt()
     monkeypatch.setattr(op_module, "load_ext", lambda: ext)
+    monkeypatch.setattr(op_module, "_stream_id", lambda device: 0)
+    op_module._workspaces.clear()
 
     # the operator insists on a GPU tensor; let CPU tensors pass for this host-logic test
     monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
@@ -200,6 +209,32 @@ def test_operator_marshalling_matches_reference_order(fake_ext):
     assert b[6].tolist() == pytest.approx(list(w.roi_range)) and b[7].tolist() == list(w.grid_size)
     assert torch.all(d.grad == 2.0) and torch.all(f.grad == 3.0)
     assert b[8].dtype == torch.float32 and b[9].dtype == torch.float32
+
+
+def test_persistent_workspace_is_prepared_once_per_shape_and_dropped_when_switched_off(fake_ext, monkeypatch):
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+
+    def step(grid=None):
+        f = x["image_feats"].clone().requires_grad_(True)
+        out = flash_bevpool(f, x["depth_params"], x["projection_matrices"], x["feature_size"], x["image_size"],
+                            x["roi_range"], x["grid_size"] if grid is None else grid)
+        out.sum().backward()
+        return fake_ext.bwd[-1]
+
+    ws = step()
+    assert ws is not None and ws.dtype == torch.uint8 and fake_ext.prepared == 1
+    assert step() is ws and fake_ext.prepared == 1                       # same shape: the same workspace
+    assert step([32, 32, 2]) is not ws and fake_ext.prepared == 2        # another grid: another workspace
+    assert len(op_module._workspaces) == 2
+    monkeypatch.setenv("FLASHBEV_WORKSPACES", "0")
+    assert step() is None                                                # per-call workspace from the allocator
+    monkeypatch.setenv("FLASHBEV_WORKSPACES", "1")
+    step([32, 32, 3])
+    assert len(op_module._workspaces) == 1                               # least recently used ones are dropped
+    monkeypatch.setenv("FLASHBEV_WORKSPACE_MB", "0.001")
+    op_module._workspaces.clear()
+    assert step() is None                                                # larger than the limit: not kept
 
 
 def test_wrapper_puts_feats_first_and_skips_unneeded_grads(fake_ext):
