@@ -15,7 +15,7 @@ FBEV_F32, FBEV_F16, FBEV_BF16 = 0, 1, 2
 FBEV_GAUSSIAN, FBEV_LAPLACE, FBEV_CATEGORICAL = 0, 1, 2
 FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
-EXPORTS = ("fbev_forward", "fbev_backward", "fbev_backward_gather", "fbev_backward_gather_static",
+EXPORTS = ("fbev_forward", "fbev_geometry_cache_bytes", "fbev_geometry_cache_build", "fbev_forward_cached", "fbev_backward", "fbev_backward_gather", "fbev_backward_gather_static",
            "fbev_static_scratch_bytes", "fbev_backward_persistent_workspace_bytes", "fbev_backward_workspace_init",
            "fbev_backward_gather_persistent", "fbev_backward_columns",
            "fbev_backward_columns_workspace_bytes", "fbev_backward_max_pairs",
@@ -56,6 +56,12 @@ def load() -> ctypes.CDLL:
         vp, pp = ctypes.c_void_p, ctypes.POINTER(FbevProblem)
         lib.fbev_forward.argtypes = [pp, vp, vp, vp, vp, vp, vp]
         lib.fbev_forward.restype = ctypes.c_int
+        lib.fbev_geometry_cache_bytes.argtypes = [pp]
+        lib.fbev_geometry_cache_bytes.restype = ctypes.c_size_t
+        lib.fbev_geometry_cache_build.argtypes = [pp, vp, vp, ctypes.c_size_t, vp]
+        lib.fbev_geometry_cache_build.restype = ctypes.c_int
+        lib.fbev_forward_cached.argtypes = [pp, vp, vp, vp, ctypes.c_size_t, vp, vp, vp]
+        lib.fbev_forward_cached.restype = ctypes.c_int
         lib.fbev_backward.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp]
         lib.fbev_backward.restype = ctypes.c_int
         lib.fbev_backward_gather.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp, ctypes.c_size_t, vp]
@@ -143,6 +149,21 @@ def forward(p: FbevProblem, depth_ptr: int, feats_ptr: int, proj_ptr: int, out_p
             stream: int = 0, count_ptr: Optional[int] = None) -> int:
     return load().fbev_forward(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(proj_ptr), _p(out_ptr),
                                _p(count_ptr), _p(stream))
+
+
+def geometry_cache_bytes(p: FbevProblem) -> int:
+    return int(load().fbev_geometry_cache_bytes(ctypes.byref(p)))
+
+
+def geometry_cache_build(p: FbevProblem, proj_ptr: int, cache_ptr: int, cache_bytes: int, stream: int = 0) -> int:
+    return load().fbev_geometry_cache_build(ctypes.byref(p), _p(proj_ptr), _p(cache_ptr),
+                                            ctypes.c_size_t(int(cache_bytes)), _p(stream))
+
+
+def forward_cached(p: FbevProblem, depth_ptr: int, feats_ptr: int, cache_ptr: int, cache_bytes: int, out_ptr: int,
+                   stream: int = 0, count_ptr: Optional[int] = None) -> int:
+    return load().fbev_forward_cached(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(cache_ptr),
+                                      ctypes.c_size_t(int(cache_bytes)), _p(out_ptr), _p(count_ptr), _p(stream))
 
 
 def backward(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,

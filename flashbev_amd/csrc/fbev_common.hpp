@@ -12,13 +12,14 @@ namespace {
 // call count per kernel.  Disabled (the default) it costs one relaxed atomic load per launch.
 namespace prof {
 enum Kid { kForward, kBackwardScatter, kZero, kCount, kScanChunks, kScanSums, kBackwardCells, kBackwardTexel,
-           kGeometry, kBackwardColumn, kCellCount, kPillar, kProjection, kNum };
+           kGeometry, kBackwardColumn, kCellCount, kPillar, kProjection, kForwardCached, kGeometryCache, kNum };
 const char *const kNames[kNum] = {"fbev_forward_kernel", "fbev_backward_cells_kernel<scatter>",
                                   "fbev_fill_zero_kernel", "fbev_count_kernel", "fbev_scan_chunks_kernel",
                                   "fbev_scan_sums_kernel", "fbev_backward_cells_kernel<fill>",
                                   "fbev_backward_texel_kernel", "fbev_geometry_kernel",
                                   "fbev_backward_column_kernel", "fbev_forward_kernel<count only>",
-                                  "fbev_pillar_kernel", "fbev_projection_kernel"};
+                                  "fbev_pillar_kernel", "fbev_projection_kernel", "fbev_forward_cached_kernel",
+                                  "fbev_geometry_cache_kernel"};
 struct Rec { hipEvent_t a, b; int kid; };
 std::atomic<bool> enabled{false};
 std::mutex mu;

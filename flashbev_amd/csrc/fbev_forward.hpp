@@ -5,42 +5,45 @@
 namespace {
 
 // ---------------------------------------------------------------- forward
+// How the lanes of a wavefront share the slots in phase B.
+struct LaneRole {
+    int gps;        // lane groups per slot
+    int slot, sub;  // this lane's slot and its group's index among the slot's groups
+    int lis;        // lane within the group
+    bool carrier;   // the lane belongs to a slot
+    int span;       // channels covered per pass
+};
+
+template <int VEC, int CPL>
+__device__ __forceinline__ LaneRole lane_role(const KParams &k, int lane) {
+    LaneRole r;
+    // a lane group covers the channels of one cell; when long lists leave room for few slots,
+    // several groups share a slot and take its entries in turn
+    r.gps = k.groups_per_slot;
+    const int group = lane / k.lanes_per_slot;
+    r.slot = group / r.gps;
+    r.sub = group - r.slot * r.gps;
+    r.lis = lane - group * k.lanes_per_slot;
+    r.carrier = r.slot < k.slots;
+    r.span = k.lanes_per_slot * VEC * CPL;
+    return r;
+}
+
+// Phase B of one round: every slot walks its list of kept samples (phase A left the lists, their
+// lengths and the cells in LDS) and stores its cell's row of the output.
 // STREAM: the output is stored with non-temporal stores (a template parameter: as a run-time
 // choice between two stores the compiler merges them into one ordinary store).
 template <typename T, int VEC, int CPL, bool STREAM>
-__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
-    KParams k, const T *__restrict__ depth, const T *__restrict__ feats, const float *__restrict__ proj,
-    float *__restrict__ out, float *__restrict__ count_out) {
-    extern __shared__ float4 smem[];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x >> 6;
-    const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
-    const int b = bid / k.blocks_per_batch;
-    const int blk = bid - b * k.blocks_per_batch;
-
-    const WaveLds L = block_lds_setup(k, smem, proj, b, 2);
+__device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds &L, const LaneRole &role, int b,
+                                                const T *__restrict__ feats, float *__restrict__ out,
+                                                float *__restrict__ count_out) {
     lds_counter *cnt = L.cnt;
-    float4 *lst = L.lst;
-
-    const int cells_per_wave = k.slots * k.rounds;
-    // a lane group covers the channels of one cell; when long lists leave room for few slots,
-    // several groups share a slot and take its entries in turn
-    const int gps = k.groups_per_slot;
-    const int group = lane / k.lanes_per_slot;
-    const int slot = group / gps, sub = group - slot * gps;
-    const int lis = lane - group * k.lanes_per_slot;
-    const bool carrier = slot < k.slots;
-    const int span = k.lanes_per_slot * VEC * CPL;   // channels covered per pass
+    const float4 *lst = L.lst;
+    const int gps = role.gps, slot = role.slot, sub = role.sub, lis = role.lis, span = role.span;
+    const bool carrier = role.carrier;
     constexpr int kUnitShift = VEC > 1 ? 4 : (sizeof(T) == 4 ? 2 : 1);
     const char *fbytes = reinterpret_cast<const char *>(feats);
-
-    for (int r = 0; r < k.rounds; ++r) {
-        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
-        if (q0 >= k.padded_cells) break;
-        phase_a<2, T, kModeForward>(k, L, depth, b, q0, lane);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-
+    {
         // phase A left the slot's cell in LDS: valid flag and ix | iy << 16
         const float4 mycell = L.cell[carrier ? slot : 0];
         const int ix = __float_as_int(mycell.w) & 0xffff, iy = __float_as_int(mycell.w) >> 16;
@@ -148,6 +151,185 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
                     }
                 }
             }
+        }
+    }
+}
+
+template <typename T, int VEC, int CPL, bool STREAM>
+__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
+    KParams k, const T *__restrict__ depth, const T *__restrict__ feats, const float *__restrict__ proj,
+    float *__restrict__ out, float *__restrict__ count_out) {
+    extern __shared__ float4 smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
+    const int b = bid / k.blocks_per_batch;
+    const int blk = bid - b * k.blocks_per_batch;
+
+    const WaveLds L = block_lds_setup(k, smem, proj, b, 2);
+    const LaneRole role = lane_role<VEC, CPL>(k, lane);
+    const int cells_per_wave = k.slots * k.rounds;
+    for (int r = 0; r < k.rounds; ++r) {
+        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
+        if (q0 >= k.padded_cells) break;
+        phase_a<2, T, kModeForward>(k, L, depth, b, q0, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        forward_phase_b<T, VEC, CPL, STREAM>(k, L, role, b, feats, out, count_out);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// ---------------------------------------------------------------- forward on cached geometry
+// The samples in view depend on the calibration and the grid only.  When those repeat from call to
+// call (a fixed rig at inference), fbev_geometry_cache_build keeps, per cell, the compacted list of
+// its samples in view -- 16 bytes each: the bilinear fractions, the first corner texel with the two
+// clamp flags below it, and the sample's depth along the optical axis, exactly the values the sample
+// phase computes -- and this kernel starts from those lists: no matrices, no column cull, no
+// projection, no divisions; the depth model, the weight threshold and phase B are the same code, on
+// the same values in the same order, so the results are the same bit for bit.
+// Cache layout: [256 bytes: header][B * padded_cells int32: samples in view per cell, cells in the
+// order of the tiled walk][B * padded_cells * NZ entries].
+constexpr int kCacheHeaderBytes = 256;
+constexpr int kCacheMagic = 0x46424743;      // "FBGC"
+
+__device__ __forceinline__ const int *cache_counts(const void *cache) {
+    return reinterpret_cast<const int *>(static_cast<const char *>(cache) + kCacheHeaderBytes);
+}
+__host__ __device__ inline size_t cache_entries_offset(long long cells) {
+    return (size_t)kCacheHeaderBytes + ((size_t)cells * sizeof(int) + 255) / 256 * 256;
+}
+
+// Sample phase on cached geometry: lanes = the cached samples of the round's cells, densely packed.
+template <typename T>
+__device__ __forceinline__ void phase_a_cached(const KParams &k, const WaveLds &L, const T *__restrict__ depth,
+                                               const int *__restrict__ counts, const float4 *__restrict__ entries,
+                                               int b, int q0, int lane) {
+    if (lane < 16) L.cnt[lane] = 0;
+    // lane s < slots: its cell, the number of cached samples, and where they start among the round's
+    int mine_n = 0;
+    if (lane < k.slots) {
+        int ix = 0, iy = 0;
+        const bool ok = cell_of(k, q0 + lane, ix, iy);
+        mine_n = ok ? counts[(size_t)b * k.padded_cells + q0 + lane] : 0;
+        L.cell[lane] = make_float4(0.0f, 0.0f, ok ? 1.0f : 0.0f, __int_as_float(ix | (iy << 16)));
+    }
+    int incl = mine_n;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        const int other = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += other;
+    }
+    const int total = __shfl(incl, 15, kWave);        // slots <= 16; lanes past the slots carry 0
+    const int my_start = incl - mine_n;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const float4 *base = entries + ((size_t)b * k.padded_cells + q0) * k.NZ;
+    for (int jb = 0; jb < total; jb += kWave) {
+        const int j = jb + lane;
+        const bool active = j < total;
+        // the slot whose range holds j: the last one that starts at or before j (empty slots start
+        // where the next one does, so later ones win)
+        int slot = 0;
+        for (int s = 1; s < k.slots; ++s) slot = (__shfl(my_start, s, kWave) <= j) ? s : slot;
+        const int first = __shfl(my_start, slot, kWave);
+        float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f);
+        int4 tx = make_int4(0, 0, 0, 0);
+        bool keep = false;
+        if (active) {
+            const float4 c = base[(size_t)slot * k.NZ + (j - first)];
+            const float du = c.x, dv = c.y;
+            const int code = __float_as_int(c.z), t00 = code >> 2;
+            const float w00 = (1.0f - du) * (1.0f - dv);
+            const float w01 = (1.0f - du) * dv;
+            const float w10 = du * (1.0f - dv);
+            const float w11 = du * dv;
+            const int t01 = t00 + ((code & 2) ? k.W : 0), t10 = t00 + (code & 1), t11 = t01 + (code & 1);
+            DepthEval e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, c.w);
+            keep = e.keep;
+            tx = make_int4(t00, t01, t10, t11);
+            w0 = make_float4(w00 * e.wgt, w01 * e.wgt, w10 * e.wgt, w11 * e.wgt);
+        }
+        const int slot_eff = active ? slot : 16 + (lane & 1);       // idle lanes: no real slot
+        const int prev_slot = __shfl_up(slot_eff, 1, kWave);
+        // the lanes of one slot are contiguous: [lo, hi)
+        const unsigned long long bm = __ballot(lane == 0 || slot_eff != prev_slot);
+        const unsigned long long m = __ballot(keep);
+        const int lo = 63 - __clzll(bm & lanemask_le(lane));
+        const unsigned long long above = lane == 63 ? 0ull : (bm & ~lanemask_le(lane));
+        const int hi = above ? __ffsll((long long)above) - 1 : kWave;
+        const unsigned long long seg = (~0ull << lo) & (hi >= 64 ? ~0ull : ((1ull << hi) - 1ull));
+        const int prefix = __popcll(m & seg & lanemask_lt(lane));
+        const int old = active ? L.cnt[slot] : 0;
+        if (keep) {
+            float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * 2;
+            e[0] = w0;
+            e[1] = make_float4(__int_as_float(tx.x * k.row_units), __int_as_float(tx.y * k.row_units),
+                               __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
+        }
+        if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
+    }
+}
+
+template <typename T, int VEC, int CPL, bool STREAM>
+__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_cached_kernel(
+    KParams k, const T *__restrict__ depth, const T *__restrict__ feats, const void *__restrict__ cache,
+    float *__restrict__ out, float *__restrict__ count_out) {
+    extern __shared__ float4 smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
+    const int b = bid / k.blocks_per_batch;
+    const int blk = bid - b * k.blocks_per_batch;
+    const WaveLds L = wave_lds_view(k, smem, 2);
+    const LaneRole role = lane_role<VEC, CPL>(k, lane);
+    const int *counts = cache_counts(cache);
+    const float4 *entries = reinterpret_cast<const float4 *>(static_cast<const char *>(cache) +
+                                                             cache_entries_offset((long long)k.B * k.padded_cells));
+    const int cells_per_wave = k.slots * k.rounds;
+    for (int r = 0; r < k.rounds; ++r) {
+        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
+        if (q0 >= k.padded_cells) break;
+        phase_a_cached<T>(k, L, depth, counts, entries, b, q0, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        forward_phase_b<T, VEC, CPL, STREAM>(k, L, role, b, feats, out, count_out);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// Builds the cache: the sample phase with the depth model left out (every sample in view is
+// listed), then each slot's list is copied out behind its cell's count.
+__global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_geometry_cache_kernel(KParams k, const float *__restrict__ proj,
+                                                                                   void *__restrict__ cache) {
+    extern __shared__ float4 smem[];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
+    const int b = bid / k.blocks_per_batch;
+    const int blk = bid - b * k.blocks_per_batch;
+    const WaveLds L = block_lds_setup(k, smem, proj, b, 1);
+    int *counts = reinterpret_cast<int *>(static_cast<char *>(cache) + kCacheHeaderBytes);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        // what the lists were built for, for whoever inspects a cache: the library never reads it back
+        int *h = static_cast<int *>(cache);
+        h[0] = kCacheMagic; h[1] = k.B; h[2] = k.N; h[3] = k.H; h[4] = k.W; h[5] = k.gx; h[6] = k.gy; h[7] = k.gz;
+        h[8] = k.padded_cells; h[9] = k.NZ;
+    }
+    float4 *entries = reinterpret_cast<float4 *>(static_cast<char *>(cache) +
+                                                 cache_entries_offset((long long)k.B * k.padded_cells));
+    const int cells_per_wave = k.slots * k.rounds;
+    for (int r = 0; r < k.rounds; ++r) {
+        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
+        if (q0 >= k.padded_cells) break;
+        phase_a<1, float, kModeCache>(k, L, nullptr, b, q0, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int s = 0; s < k.slots && q0 + s < k.padded_cells; ++s) {
+            const size_t cell = (size_t)b * k.padded_cells + q0 + s;
+            const int n = L.cnt[s];
+            if (lane == 0) counts[cell] = n;
+            for (int i = lane; i < n; i += kWave) entries[cell * k.NZ + i] = L.lst[(size_t)s * k.list_cap + i];
         }
         __builtin_amdgcn_wave_barrier();
     }

@@ -230,6 +230,43 @@ int dispatch_forward(const fbev_problem *p, const Plan &pl, const void *depth, c
 }
 
 template <typename T, int VEC>
+int launch_forward_cached(const Plan &pl, const void *depth, const void *feats, const void *cache, float *out,
+                          float *cnt, hipStream_t st) {
+    dim3 grid(pl.k.n_blocks), block(kWave * pl.k.waves);
+    const T *d = static_cast<const T *>(depth);
+    const T *f = static_cast<const T *>(feats);
+    prof::Scope timer(prof::kForwardCached, st);
+    const bool stream = VEC > 1 && (long long)pl.k.B * pl.k.gy * pl.k.gx * pl.k.C * 4 > kStreamOutputFrom;
+    auto launch = [&](auto kernel) {
+        if (!lds_opt_in(kernel, pl.lds_fwd)) return false;
+        hipLaunchKernelGGL(kernel, grid, block, pl.lds_fwd, st, pl.k, d, f, cache, out, cnt);
+        return true;
+    };
+    bool ok;
+    if (stream) {
+        constexpr bool S = VEC > 1;
+        ok = pl.cpl == 1 ? launch(fbev_forward_cached_kernel<T, VEC, 1, S>)
+                         : (pl.cpl == 2 ? launch(fbev_forward_cached_kernel<T, VEC, 2, S>)
+                                        : launch(fbev_forward_cached_kernel<T, VEC, 4, S>));
+    } else {
+        ok = pl.cpl == 1 ? launch(fbev_forward_cached_kernel<T, VEC, 1, false>)
+                         : (pl.cpl == 2 ? launch(fbev_forward_cached_kernel<T, VEC, 2, false>)
+                                        : launch(fbev_forward_cached_kernel<T, VEC, 4, false>));
+    }
+    if (!ok) return FBEV_ERR_LAUNCH;
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+// bytes of a geometry cache; 0 when the problem is outside its limits
+size_t geometry_cache_bytes(const fbev_problem *p) {
+    const long long tiles = (long long)((p->grid_x + kTile - 1) / kTile) * ((p->grid_y + kTile - 1) / kTile);
+    const long long cells = (long long)p->batch * tiles * 64;
+    // a cached first-corner texel shares its word with the two clamp flags
+    if ((long long)p->batch * p->num_cams * p->feat_h * p->feat_w >= (1ll << 29)) return 0;
+    return cache_entries_offset(cells) + (size_t)cells * p->num_cams * p->grid_z * sizeof(float4);
+}
+
+template <typename T, int VEC>
 int launch_columns(const Plan &pl, const ColParams &cp, size_t lds, const float *go, const void *depth,
                    const void *feats, const float *proj, const float *count, float *dd, float *df, hipStream_t st) {
     auto kernel = fbev_backward_column_kernel<T, VEC>;
@@ -532,6 +569,63 @@ int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, co
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kCellPassWaves, 4);
     if (rc != FBEV_OK) return rc;
     return dispatch_forward(p, pl, depth, feats, proj, out, count_out, static_cast<hipStream_t>(stream));
+}
+
+size_t fbev_geometry_cache_bytes(const fbev_problem *p) {
+    if (validate(p, false) != FBEV_OK) return 0;
+    return geometry_cache_bytes(p);
+}
+
+int fbev_geometry_cache_build(const fbev_problem *p, const float *proj, void *cache, size_t cache_bytes, void *stream) {
+    int rc = validate(p, false);
+    if (rc != FBEV_OK) return rc;
+    if (!proj || !cache) return FBEV_ERR_NULL;
+    if ((uintptr_t)proj % 4 || (uintptr_t)cache % 16) return FBEV_ERR_ALIGNMENT;
+    const size_t need = geometry_cache_bytes(p);
+    if (need == 0) return FBEV_ERR_TOO_LARGE;
+    if (cache_bytes < need) return FBEV_ERR_SHAPE;
+    fbev_problem q = *p;      // the lists depend on the geometry only
+    q.channels = 4; q.in_dtype = FBEV_F32; q.depth_distribution = FBEV_GAUSSIAN; q.depth_bins = 2;
+    q.reduction = FBEV_REDUCE_MEAN;
+    Plan pl;
+    rc = make_plan(&q, true, &pl, kCellPassWaves, 4);
+    if (rc != FBEV_OK) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t lds = pl.lds_fwd;         // sized for two-word entries: more than the one-word lists need
+    if (!lds_opt_in(fbev_geometry_cache_kernel, lds)) return FBEV_ERR_LAUNCH;
+    prof::Scope timer(prof::kGeometryCache, st);
+    hipLaunchKernelGGL(fbev_geometry_cache_kernel, dim3(pl.k.n_blocks), dim3(kWave * pl.k.waves), lds, st, pl.k, proj,
+                       cache);
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+int fbev_forward_cached(const fbev_problem *p, const void *depth, const void *feats, const void *cache,
+                        size_t cache_bytes, float *out, float *count_out, void *stream) {
+    int rc = validate(p, true);
+    if (rc != FBEV_OK) return rc;
+    if (!depth || !feats || !cache || !out) return FBEV_ERR_NULL;
+    const int es = elem_size(p->in_dtype);
+    if ((uintptr_t)depth % es || (uintptr_t)feats % es || (uintptr_t)cache % 16 || (uintptr_t)out % 4 ||
+        (uintptr_t)count_out % 4)
+        return FBEV_ERR_ALIGNMENT;
+    const size_t need = geometry_cache_bytes(p);
+    if (need == 0) return FBEV_ERR_TOO_LARGE;
+    if (cache_bytes < need) return FBEV_ERR_SHAPE;
+    Plan pl;
+    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kCellPassWaves, 4);
+    if (rc != FBEV_OK) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (p->in_dtype) {
+        case FBEV_F32:
+            return pl.vec == 4 ? launch_forward_cached<float, 4>(pl, depth, feats, cache, out, count_out, st)
+                               : launch_forward_cached<float, 1>(pl, depth, feats, cache, out, count_out, st);
+        case FBEV_F16:
+            return pl.vec == 8 ? launch_forward_cached<__half, 8>(pl, depth, feats, cache, out, count_out, st)
+                               : launch_forward_cached<__half, 1>(pl, depth, feats, cache, out, count_out, st);
+        default:
+            return pl.vec == 8 ? launch_forward_cached<bf16_raw, 8>(pl, depth, feats, cache, out, count_out, st)
+                               : launch_forward_cached<bf16_raw, 1>(pl, depth, feats, cache, out, count_out, st);
+    }
 }
 
 int fbev_backward(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,

@@ -32,26 +32,33 @@ __device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots * 
 __device__ __forceinline__ int lds_cand_f4(const KParams &k) { return (k.slots * k.NZ + 3) / 4; }
 __device__ __forceinline__ int lds_z_f4(const KParams &k) { return (k.gz + 3) / 4; }
 
-// Stage the block's matrices, the column table and the height table; returns the wavefront's view.  Ends with a
-// barrier.
-__device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *smem, const float *__restrict__ proj,
-                                                   int b, int entry_f4) {
+// The wavefront's view of the block's LDS (pointers only).
+__device__ __forceinline__ WaveLds wave_lds_view(const KParams &k, float4 *smem, int entry_f4) {
     WaveLds L;
-    float *Pm = reinterpret_cast<float *>(smem);
-    int *dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
     const int dec_f4 = lds_dec_f4(k), cand_f4 = lds_cand_f4(k), cols = k.slots * k.N;
     const int per_wave_f4 = 4 + 16 + cols + dec_f4 + cand_f4 + k.slots * k.list_cap * entry_f4;
-    float *zt = reinterpret_cast<float *>(smem + lds_p_f4(k) + dec_f4);
     float4 *wbase = smem + lds_p_f4(k) + dec_f4 + lds_z_f4(k) + (threadIdx.x >> 6) * per_wave_f4;
-    L.Pm = Pm;
-    L.dec = dec;
-    L.zt = zt;
+    L.Pm = reinterpret_cast<float *>(smem);
+    L.dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
+    L.zt = reinterpret_cast<float *>(smem + lds_p_f4(k) + dec_f4);
     L.cnt = (lds_counter *)reinterpret_cast<int *>(wbase);
     L.cell = wbase + 4;
     L.col = wbase + 20;
     L.alive = reinterpret_cast<int *>(wbase + 20 + cols);
     L.cand = reinterpret_cast<unsigned *>(wbase + 20 + cols + dec_f4);
     L.lst = wbase + 20 + cols + dec_f4 + cand_f4;
+    return L;
+}
+
+// Stage the block's matrices, the column table and the height table; returns the wavefront's view.  Ends with a
+// barrier.
+__device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *smem, const float *__restrict__ proj,
+                                                   int b, int entry_f4) {
+    const WaveLds L = wave_lds_view(k, smem, entry_f4);
+    float *Pm = reinterpret_cast<float *>(smem);
+    int *dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
+    float *zt = reinterpret_cast<float *>(smem + lds_p_f4(k) + lds_dec_f4(k));
+    const int cols = k.slots * k.N;
     for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
         Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
@@ -68,12 +75,13 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 //             word 1: where the four texels' feature rows start, in address units (texel index
 //                     ((b*N+n)*H + v)*W + u times KParams::row_units) as int bits (t00, t01, t10, t11):
 //                     the gather loop then forms an address with one shift-add, not a 64-bit multiply
+//   cache     one word: du, dv, t00 << 2 | (u1 != u0) | (v1 != v0) << 1, depth along the optical axis
 //   backward  word 0: du, dv, t00, (u1 != u0) | (v1 != v0) << 1 -- the four weights and texels
 //                     follow from these exactly as phase A computed them.  Inverse map: t00 << 2 with
 //                     the two flags below it, and in the fourth place the position of the sample's
 //                     pair in the pair array (sorted by first corner texel), or -1 if the array is full
 //             word 1: wgt, a, b, (k0 | k1 << 16)
-enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeFillRuns = 4 };
+enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeFillRuns = 4, kModeCache = 5 };
 
 // Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
 // pixel coordinate misses the image by more than this fraction, far beyond any rounding of
@@ -201,10 +209,20 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                 int t01 = (rowbase + g.v1) * k.W + g.u0;
                 int t10 = (rowbase + g.v0) * k.W + g.u1;
                 int t11 = (rowbase + g.v1) * k.W + g.u1;
-                DepthEval e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
+                DepthEval e;
+                if (MODE == kModeCache) {
+                    e.keep = true;       // every sample in view is listed; the depth model comes later
+                    e.wgt = e.a = e.b = 0.0f;
+                    e.k0 = e.k1 = 0;
+                } else {
+                    e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
+                }
                 keep = e.keep;
                 tx = make_int4(t00, t01, t10, t11);
-                if (BACKWARD) {
+                if (MODE == kModeCache) {
+                    const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
+                    w0 = make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), g.depth);
+                } else if (BACKWARD) {
                     const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
                     w0 = FILLING ? make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1))
                                            : make_float4(g.du, g.dv, __int_as_float(t00), __int_as_float(fl));
@@ -251,9 +269,10 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         if (keep) {
             float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
             e[0] = w0;
-            e[1] = BACKWARD ? w2
-                            : make_float4(__int_as_float(tx.x * k.row_units), __int_as_float(tx.y * k.row_units),
-                                          __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
+            if (ENTRY_F4 > 1)
+                e[1] = BACKWARD ? w2
+                                : make_float4(__int_as_float(tx.x * k.row_units), __int_as_float(tx.y * k.row_units),
+                                              __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
         }
         if (MODE == kModeFill && keep) {
             // claim the sample's position in the list of its first corner texel

@@ -162,7 +162,8 @@ void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &ima
                            double voxel_z_min, at::Tensor out, int64_t total_threads, int depth_distribution,
                            bool use_shared_memory, bool optimize_z_precompute, bool use_warp_kernel,
                            bool use_vectorized_load, float epsilon, float depth_weight_threshold,
-                           float depth_min, float depth_step, int reduction, std::optional<at::Tensor> count_out) {
+                           float depth_min, float depth_step, int reduction, std::optional<at::Tensor> count_out,
+                           std::optional<at::Tensor> geometry_cache) {
     (void)use_shared_memory; (void)optimize_z_precompute; (void)use_warp_kernel; (void)use_vectorized_load;
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
@@ -185,9 +186,51 @@ void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &ima
     }
     DeviceScope scope(depth_params.get_device());
     hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
+    if (geometry_cache.has_value() && geometry_cache->defined()) {
+        // lists built by build_geometry_cache for these matrices and this grid: same result, less work
+        check_dev(*geometry_cache, depth_params, "geometry_cache");
+        TORCH_CHECK(geometry_cache->scalar_type() == at::kByte, "flashbevpool_ext: geometry_cache must be a uint8 tensor");
+        raise_on(fbev_forward_cached(&p, depth_params.data_ptr(), image_feats.data_ptr(), geometry_cache->data_ptr(),
+                                     (size_t)geometry_cache->numel(), out.data_ptr<float>(), cnt, st),
+                 "fbev_forward_cached");
+        return;
+    }
     raise_on(fbev_forward(&p, depth_params.data_ptr(), image_feats.data_ptr(), projection_matrices.data_ptr<float>(),
                           out.data_ptr<float>(), cnt, st),
              "fbev_forward");
+}
+
+// The per-cell lists of samples in view for these matrices and this grid (fbev_geometry_cache_build),
+// as a uint8 tensor to hand to flash_bevpool_forward while calibration and grid stay the same.
+at::Tensor build_geometry_cache(const at::Tensor &projection_matrices, int64_t feat_h, int64_t feat_w, int64_t image_h,
+                                int64_t image_w, std::vector<int64_t> grid_size, std::vector<double> voxel_min,
+                                std::vector<double> voxel_size, float epsilon) {
+    TORCH_CHECK(projection_matrices.is_cuda() && projection_matrices.is_contiguous() &&
+                    projection_matrices.scalar_type() == at::kFloat && projection_matrices.dim() == 4 &&
+                    (projection_matrices.size(2) == 3 || projection_matrices.size(2) == 4) &&
+                    projection_matrices.size(3) == 4,
+                "flashbevpool_ext: projection_matrices must be a contiguous float32 GPU tensor [B,N,3|4,4]");
+    TORCH_CHECK(grid_size.size() == 3 && voxel_min.size() == 3 && voxel_size.size() == 3,
+                "flashbevpool_ext: grid_size, voxel_min and voxel_size need 3 entries each");
+    fbev_problem p{};
+    p.batch = (int32_t)projection_matrices.size(0);
+    p.num_cams = (int32_t)projection_matrices.size(1);
+    p.feat_h = (int32_t)feat_h; p.feat_w = (int32_t)feat_w;
+    p.image_h = (int32_t)image_h; p.image_w = (int32_t)image_w;
+    p.grid_x = (int32_t)grid_size[0]; p.grid_y = (int32_t)grid_size[1]; p.grid_z = (int32_t)grid_size[2];
+    for (int a = 0; a < 3; ++a) { p.voxel_min[a] = voxel_min[a]; p.voxel_size[a] = voxel_size[a]; }
+    p.epsilon = epsilon;
+    p.channels = 1; p.depth_bins = 2;
+    p.proj_stride = (int32_t)(projection_matrices.size(2) * 4);
+    const size_t bytes = fbev_geometry_cache_bytes(&p);
+    TORCH_CHECK(bytes > 0, "flashbevpool_ext: no geometry cache for this problem (sizes must be positive and "
+                           "B*N*H*W below 2^29)");
+    at::Tensor cache = at::empty({(int64_t)bytes}, projection_matrices.options().dtype(at::kByte));
+    DeviceScope scope(projection_matrices.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(projection_matrices.get_device()).stream();
+    raise_on(fbev_geometry_cache_build(&p, projection_matrices.data_ptr<float>(), cache.data_ptr(), bytes, st),
+             "fbev_geometry_cache_build");
+    return cache;
 }
 
 // Same positional order as the reference's flash_bevpool_backward
@@ -442,7 +485,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("out"), py::arg("total_threads"), py::arg("depth_distribution"), py::arg("use_shared_memory"),
           py::arg("optimize_z_precompute"), py::arg("use_warp_kernel"), py::arg("use_vectorized_load"),
           py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f, py::arg("depth_min") = 1.0f,
-          py::arg("depth_step") = 1.0f, py::arg("reduction") = 0, py::arg("count_out") = py::none());
+          py::arg("depth_step") = 1.0f, py::arg("reduction") = 0, py::arg("count_out") = py::none(),
+          py::arg("geometry_cache") = py::none());
+    m.def("build_geometry_cache", &build_geometry_cache,
+          "per-cell lists of the samples in view, for flash_bevpool_forward(..., geometry_cache=...)",
+          py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
+          py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);
     m.def("flash_bevpool_backward", &flash_bevpool_backward, "fused camera->BEV pooling, backward",
           py::arg("out_grad"), py::arg("depth_params"), py::arg("image_feats"), py::arg("projection_matrices"),
           py::arg("feature_size"), py::arg("image_size"), py::arg("roi_range"), py::arg("grid_size"),

@@ -183,7 +183,8 @@ class FlashBEVPool(torch.autograd.Function):
     def forward(ctx, depth_params, image_feats, projection_matrices, feature_size, image_size,
                 roi_range, grid_size, depth_distribution=0, use_shared_memory=True,
                 optimize_z_precompute=True, use_warp_kernel=False, use_vectorized_load=False,
-                epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=None, reduction="mean"):
+                epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=None, reduction="mean",
+                geometry_cache=None):
         ext = load_ext()
         if not (isinstance(image_feats, torch.Tensor) and image_feats.is_cuda):
             raise RuntimeError("flash_bevpool: image_feats must be a tensor on a ROCm GPU; "
@@ -226,7 +227,7 @@ class FlashBEVPool(torch.autograd.Function):
             vsize[0], vsize[1], vsize[2], vmin[0], vmin[1], vmin[2], out, out.numel(),
             depth_distribution, bool(use_shared_memory), bool(optimize_z_precompute),
             bool(use_warp_kernel), bool(use_vectorized_load), float(epsilon),
-            float(depth_weight_threshold), d_min, d_step, red, counts)
+            float(depth_weight_threshold), d_min, d_step, red, counts, geometry_cache)
 
         ctx.save_for_backward(depth_params, image_feats, projection_matrices)
         ctx.counts = counts
@@ -269,23 +270,46 @@ class FlashBEVPool(torch.autograd.Function):
             except Exception:
                 _workspaces.pop(key, None)       # a failed call leaves a persistent workspace undefined
                 raise
-        return (depth_params_grad, image_feats_grad) + (None,) * 14
+        return (depth_params_grad, image_feats_grad) + (None,) * 15
 
 
 def flash_bevpool(image_feats, depth_params, projection_matrices, feature_size, image_size,
                   roi_range, grid_size, depth_distribution=0, use_shared_memory=True,
                   optimize_z_precompute=True, use_warp_kernel=False, use_vectorized_load=False,
-                  epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=None, reduction="mean"):
+                  epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=None, reduction="mean",
+                  geometry_cache=None):
     """Keyword-friendly wrapper; note ``image_feats`` comes first here and second in
     ``FlashBEVPool.apply`` (as in flashbev/flashbevpool/flash_bevpool.py:139-178).
 
     image_feats [B,N,H,W,C], depth_params [B,N,H,W,2] (mean, sigma) or [B,N,H,W,D] for the
     categorical model, projection_matrices [B,N,3|4,4], feature_size [B,N,2], image_size
     [2] (rows, cols), roi_range [6] (xmin,xmax,ymin,ymax,zmin,zmax), grid_size [3]
-    (x,y,z).  Returns [B, Y, X, C] float32.
+    (x,y,z).  Returns [B, Y, X, C] float32.  ``geometry_cache`` (from ``build_geometry_cache`` for the same
+    matrices, sizes, grid and epsilon) lets the forward skip the projection; the result is the same bit for bit.
     """
     return FlashBEVPool.apply(depth_params, image_feats, projection_matrices, feature_size,
                               image_size, roi_range, grid_size, depth_distribution,
                               use_shared_memory, optimize_z_precompute, use_warp_kernel,
                               use_vectorized_load, epsilon, depth_weight_threshold, depth_range,
-                              reduction)
+                              reduction, geometry_cache)
+
+
+def build_geometry_cache(projection_matrices, feature_size, image_size, roi_range, grid_size, epsilon=1e-6):
+    """Per-cell lists of the samples in view for one calibration and grid, as an opaque uint8 tensor
+    for ``flash_bevpool(..., geometry_cache=...)``.  Worth building when ``projection_matrices``
+    repeat from call to call (a fixed rig at inference); it must be rebuilt whenever the matrices,
+    the feature-map or image size, the grid, the region of interest or ``epsilon`` change -- nothing
+    checks that.  ``feature_size`` is (H, W) of the feature maps (a pair, or the operator's [B,N,2]
+    tensor).  Size: 16 bytes per (cell, camera, height bin) sample slot."""
+    ext = load_ext()
+    if isinstance(feature_size, torch.Tensor):
+        fs = feature_size.reshape(-1).tolist() if feature_size.device.type == "cpu" else _device_values(feature_size)
+    else:
+        fs = [int(v) for row in feature_size for v in (row if hasattr(row, "__iter__") else [row])]
+    H, W = int(fs[0]), int(fs[1])
+    grid = tuple(int(v) for v in _host_values(grid_size, 3, "grid_size"))
+    image = tuple(int(v) for v in _host_values(image_size, 2, "image_size"))
+    roi = tuple(float(v) for v in _host_values(roi_range, 6, "roi_range"))
+    vmin, vsize = voxel_geometry(roi, grid)
+    return ext.build_geometry_cache(projection_matrices.contiguous().float(), H, W, image[0], image[1], list(grid),
+                                    vmin, vsize, float(epsilon))

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 7
+#define FBEV_ABI_VERSION 8
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -90,6 +90,28 @@ typedef struct fbev_problem {
  */
 int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, const float *proj,
                  float *out, float *count_out, void *stream);
+
+/*
+ * Forward on cached geometry.  Which samples are in view, and their bilinear corners and fractions,
+ * depend only on the projection matrices, the feature-map and image sizes and the grid: when those
+ * repeat from call to call (a fixed rig at inference) the lists can be built once and every later
+ * forward starts from them, skipping the column cull, the projection and its divisions (about a
+ * third of the forward at the large configurations).  The cache is caller-owned device memory of
+ * fbev_geometry_cache_bytes(p) bytes (0: outside the limits, B*N*H*W >= 2^29), 16-byte aligned:
+ * per BEV cell the number of samples in view and up to N * grid_z 16-byte records (du, dv, first
+ * corner texel with the two clamp flags, depth along the optical axis), i.e.
+ * B * ceil(gx/8) * ceil(gy/8) * 64 * (4 + 16 * N * grid_z) bytes.  fbev_geometry_cache_build fills it
+ * (p->channels, in_dtype and the depth fields are ignored); fbev_forward_cached is fbev_forward with
+ * the cache in place of the matrices and gives the same result bit for bit.  The caller rebuilds
+ * the cache whenever proj, the sizes, the grid, the region of interest or epsilon change; nothing
+ * checks that.  The optional cached workspace keyed by geometry has no counterpart in the reference,
+ * which recomputes the projection per channel thread (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:102-159).
+ */
+size_t fbev_geometry_cache_bytes(const fbev_problem *p);
+int fbev_geometry_cache_build(const fbev_problem *p, const float *proj, void *cache, size_t cache_bytes,
+                              void *stream);
+int fbev_forward_cached(const fbev_problem *p, const void *depth, const void *feats, const void *cache,
+                        size_t cache_bytes, float *out, float *count_out, void *stream);
 
 /*
  * Backward: the exact gradients of fbev_forward.  With accumulate != 0 they are ADDED to

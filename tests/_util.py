@@ -76,6 +76,31 @@ def capi_forward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN
     return (out, cnt) if with_count else out
 
 
+def capi_geometry_cache(x, w, dist=1, eps=1e-6):
+    """A geometry cache for a workload's matrices, built through the C ABI (a uint8 tensor)."""
+    p = problem_for(x, w, dist, 1e-6, eps)
+    nbytes = capi.geometry_cache_bytes(p)
+    assert nbytes > 0
+    cache = torch.empty(nbytes, dtype=torch.uint8, device=x["image_feats"].device).fill_(0xA5)
+    capi.check(capi.geometry_cache_build(p, x["projection_matrices"].data_ptr(), cache.data_ptr(), nbytes,
+                                         torch.cuda.current_stream().cuda_stream), "fbev_geometry_cache_build")
+    torch.cuda.synchronize()
+    return cache
+
+
+def capi_forward_cached(x, w, dist, cache, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, with_count=False):
+    """capi_forward on cached geometry."""
+    p = problem_for(x, w, dist, thr, eps, reduction)
+    dev = x["image_feats"].device
+    out = torch.full((p.batch, p.grid_y, p.grid_x, p.channels), float("nan"), dtype=torch.float32, device=dev)
+    cnt = torch.full((p.batch, p.grid_y, p.grid_x), float("nan"), dtype=torch.float32, device=dev) if with_count else None
+    capi.check(capi.forward_cached(p, x["depth_params"].data_ptr(), x["image_feats"].data_ptr(), cache.data_ptr(),
+                                   cache.numel(), out.data_ptr(), torch.cuda.current_stream().cuda_stream,
+                                   cnt.data_ptr() if with_count else None), "fbev_forward_cached")
+    torch.cuda.synchronize()
+    return (out, cnt) if with_count else out
+
+
 def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, want=(True, True),
                   mode="scatter", pair_capacity=None):
     """Backward through the C ABI.  mode "scatter" = fbev_backward, "gather" = fbev_backward_gather

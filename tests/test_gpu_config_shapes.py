@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 import torch
 
+from flashbev_amd import capi
 from flashbev_amd.workloads import WORKLOADS, make_inputs
 from oracle import c_oracle
 from tests import _util as U
@@ -92,3 +93,53 @@ def test_backward_against_the_oracle_at_the_configurations_own_shape(name, dist,
     for got, ref, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
         bad, maxabs, ratio = U.violations(got.cpu().numpy(), ref)
         assert bad == 0, (what, bad, maxabs, ratio)
+
+
+CACHED_CASES = [("cfg1_tiny", None, 0), ("cfg2_surround", None, 1), ("cfg2_surround", None, 2), ("cfg3_zsweep", 12, 1),
+                ("cfg4_hires", None, 1), ("cfg4_hires", None, 2), ("cfg5_train", None, 0)]
+
+
+@pytest.mark.parametrize("name,gz,dist", CACHED_CASES)
+def test_forward_on_cached_geometry_equals_the_forward_bit_for_bit_and_the_oracle(name, gz, dist):
+    """The cached and the uncached forward run the depth model and the accumulation on the same values
+    in the same order: identical outputs and counts; both are checked against the oracle, and the
+    cache's per-cell counts against the oracle's number of samples in view."""
+    w = workload(name, gz)
+    x = make_inputs(w, MODEL[dist], device="cuda")
+    cache = U.capi_geometry_cache(x, w, dist)
+    for thr in (1e-6, 0.0):
+        out, cnt = U.capi_forward(x, w, dist, thr, with_count=True)
+        got, got_cnt = U.capi_forward_cached(x, w, dist, cache, thr, with_count=True)
+        assert torch.equal(got, out) and torch.equal(got_cnt, cnt)
+    want = U.oracle_forward(x, w, dist, 0.0)
+    bad, maxabs, ratio = U.violations(got.cpu().numpy(), want)
+    assert bad == 0, (bad, maxabs, ratio)
+    # the header and the counts of the cache itself
+    head = cache[:40].view(torch.int32).cpu().tolist()
+    gx, gy, nz = w.grid_size
+    assert head[0] == 0x46424743 and head[1:8] == [w.batch, w.num_cams, w.feat_hw[0], w.feat_hw[1], gx, gy, nz]
+    if dist != 2:
+        # threshold 0 keeps every sample in view under the parametric models: the cache's counts, summed,
+        # are the oracle's number of valid samples
+        padded = head[8]
+        counts = cache[256:256 + 4 * w.batch * padded].view(torch.int32)
+        geo = c_oracle.geometry(x["projection_matrices"].cpu().numpy(), w.feat_hw, w.image_hw, w.roi_range, w.grid_size)
+        assert int(counts.sum().item()) == int(geo["mask"].sum())
+
+
+def test_cached_geometry_rejects_short_caches_and_follows_new_matrices():
+    w = workload("cfg2_surround")
+    x = make_inputs(w, "parametric", device="cuda")
+    p = U.problem_for(x, w, 1)
+    cache = U.capi_geometry_cache(x, w, 1)
+    out = torch.empty((1, 128, 128, 80), dtype=torch.float32, device="cuda")
+    rc = capi.forward_cached(p, x["depth_params"].data_ptr(), x["image_feats"].data_ptr(), cache.data_ptr(),
+                             cache.numel() - 16, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == -2
+    rc = capi.geometry_cache_build(p, x["projection_matrices"].data_ptr(), cache.data_ptr(), cache.numel() - 16, 0)
+    assert rc == -2
+    # a rebuilt cache follows the matrices it was built from
+    y = dict(x, projection_matrices=x["projection_matrices"].flip(1).contiguous())
+    cache2 = U.capi_geometry_cache(y, w, 1)
+    assert torch.equal(U.capi_forward_cached(y, w, 1, cache2), U.capi_forward(y, w, 1))
+    assert not torch.equal(U.capi_forward_cached(y, w, 1, cache), U.capi_forward(y, w, 1))

@@ -199,6 +199,34 @@ def test_device_resident_size_tensors_are_reused_across_calls():
     assert torch.equal(flash_bevpool(**args, **dev), want5)
 
 
+def test_operator_on_cached_geometry():
+    """flash_bevpool(..., geometry_cache=build_geometry_cache(...)): same output bit for bit, same
+    gradients (the backward does not use the cache), and a cache for another grid is refused."""
+    from flashbev_amd import build_geometry_cache
+
+    w = small(channels=32, grid_size=(40, 40, 6), dtype=torch.float16)
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    args = dict(projection_matrices=x["projection_matrices"], feature_size=x["feature_size"], image_size=x["image_size"],
+                roi_range=x["roi_range"], grid_size=x["grid_size"], depth_distribution=1)
+    cache = build_geometry_cache(x["projection_matrices"], x["feature_size"], x["image_size"], x["roi_range"],
+                                 x["grid_size"])
+    grads = []
+    outs = []
+    for gc in (None, cache):
+        f = x["image_feats"].clone().requires_grad_(True)
+        d = x["depth_params"].clone().requires_grad_(True)
+        out = flash_bevpool(image_feats=f, depth_params=d, geometry_cache=gc, **args)
+        out.backward(x["grad_out"])
+        outs.append(out.detach())
+        grads.append((f.grad, d.grad))
+    assert torch.equal(outs[0], outs[1])
+    assert torch.allclose(grads[0][0].float(), grads[1][0].float(), rtol=1e-3, atol=1e-4)
+    assert torch.allclose(grads[0][1].float(), grads[1][1].float(), rtol=1e-3, atol=1e-4)
+    with pytest.raises(RuntimeError, match="inconsistent"):
+        flash_bevpool(image_feats=x["image_feats"], depth_params=x["depth_params"], geometry_cache=cache,
+                      **dict(args, grid_size=(48, 48, 6)))
+
+
 def test_results_are_reproducible_and_stream_ordered():
     w = WORKLOADS["cfg2_surround"]
     x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)

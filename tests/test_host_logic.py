@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in flashbev_hip.h but not exported"
     assert sorted(capi.EXPORTS) == names
-    assert lib.fbev_abi_version() == 7
+    assert lib.fbev_abi_version() == 8
     assert lib.fbev_problem_size() == ctypes.sizeof(capi.FbevProblem)
 
 
