@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_count_kernel(KPara
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
-    const int b = bid / k.blocks_per_batch;
+    const int b = batch_of(k, bid);
     const int blk = bid - b * k.blocks_per_batch;
     const WaveLds L = block_lds_setup(k, smem, proj, b, 0);
     const int cells_per_wave = k.slots * k.rounds;
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
-    const int b = bid / k.blocks_per_batch;
+    const int b = batch_of(k, bid);
     const int blk = bid - b * k.blocks_per_batch;
 
     const WaveLds L = block_lds_setup(k, smem, proj, b, EF4);
@@ -189,8 +189,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     const int cells_per_wave = k.slots * k.rounds;
     // lane groups of lanes_per_slot lanes; the groups_per_slot groups of a slot take its entries in turn
     const int gps = k.groups_per_slot;
-    const int group = lane / k.lanes_per_slot;
-    const int slot = group / gps, sub = group - slot * gps;
+    const int group = (int)(((unsigned)lane * k.lps_magic) >> 16);       // lane / lanes_per_slot
+    const int slot = (int)(((unsigned)group * k.gps_magic) >> 16), sub = group - slot * gps;
     const int lis = lane - group * k.lanes_per_slot;
     const bool carrier = slot < k.slots;
     const int span = k.lanes_per_slot * VEC * CPL;
@@ -208,8 +208,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     // The depth gradient travels with the pairs when one channel pass sees the whole of G and
     // the pair's first word has room for the depth bin; otherwise it is added with atomics here.
     const bool fold = FILL && need_G && k.C <= span && k.bin_bits >= 0;
-    constexpr int kUnitShift = VEC > 1 ? 4 : (sizeof(T) == 4 ? 2 : 1);
+    // a feature row starts at a 32-bit byte offset from the tensor's base: uniform base + 32-bit lane offset
     const char *fbytes = reinterpret_cast<const char *>(feats);
+    auto row_at = [&](unsigned byte_offset) { return reinterpret_cast<const T *>(fbytes + byte_offset); };
     const unsigned row_step_v = (unsigned)(k.W * k.row_units);      // one feature-map row down
 
     for (int r = 0; r < k.rounds; ++r) {
@@ -273,7 +274,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 const float w00 = (1.0f - du) * (1.0f - dv), w01 = (1.0f - du) * dv, w10 = du * (1.0f - dv), w11 = du * dv;
                 const int t00 = entry_texel(geo), fl = entry_flags(geo);
                 const int su = fl & 1, sv = (fl & 2) ? k.W : 0;
-                // feature rows in address units: one 32-bit multiply and three adds, then a shift-add each
+                // feature rows as byte offsets: one 32-bit multiply and three adds, then one add each
                 const unsigned r00 = (unsigned)t00 * (unsigned)k.row_units;
                 const unsigned r01 = r00 + ((fl & 2) ? row_step_v : 0u);
                 const unsigned r10 = r00 + ((fl & 1) ? (unsigned)k.row_units : 0u), r11 = r01 + (r10 - r00);
@@ -286,11 +287,12 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                     const int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
                     if (ch < k.C) {
                         if (need_G) {
+                            const unsigned chb = (unsigned)ch * (unsigned)sizeof(T);
                             float f00[VEC], f01[VEC], f10[VEC], f11[VEC];
-                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r00 << kUnitShift)) + ch, f00);
-                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r01 << kUnitShift)) + ch, f01);
-                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r10 << kUnitShift)) + ch, f10);
-                            VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)r11 << kUnitShift)) + ch, f11);
+                            VecLoad<T, VEC>::ld(row_at(r00 + chb), f00);
+                            VecLoad<T, VEC>::ld(row_at(r01 + chb), f01);
+                            VecLoad<T, VEC>::ld(row_at(r10 + chb), f10);
+                            VecLoad<T, VEC>::ld(row_at(r11 + chb), f11);
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) {
                                 const float f = __builtin_fmaf(w11, f11[v], __builtin_fmaf(w10, f10[v],

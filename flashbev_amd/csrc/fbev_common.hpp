@@ -95,7 +95,11 @@ struct KParams {
     int n_blocks;
     int waves;           // wavefronts per block of the cell-centric kernels
     int bin_bits;        // a pair's first word is cell << bin_bits | depth bin; -1: the word cannot hold both
-    int row_units;       // a texel's feature row in address units: 16 bytes on the vector paths, else one element
+    int row_units;       // bytes of a texel's feature row (C * element size): rows are addressed by 32-bit byte offsets
+    unsigned tiles_x_magic;   // tile / tiles_x == umulhi(tile, tiles_x_magic) for every tile of the walk
+    unsigned lps_magic, gps_magic;   // lane / lanes_per_slot and group / groups_per_slot: (x * magic) >> 16 for x < 64
+    unsigned cams_magic;      // i / N == umulhi(i, cams_magic) for i < 2^16
+    unsigned bpb_magic;       // block / blocks_per_batch == umulhi(block, bpb_magic); 0: divide
     int gz_magic, gz_shift;   // i / gz == (i * gz_magic) >> gz_shift for 0 <= i < 4096
 };
 
@@ -261,7 +265,7 @@ __device__ __forceinline__ DepthEval eval_depth(const KParams &k, const T *__res
 // Cell index inside one batch element's padded 8x8-tiled walk -> (ix, iy).
 __device__ __forceinline__ bool cell_of(const KParams &k, int q, int &ix, int &iy) {
     int tile = q >> 6, l = q & 63;
-    int ty = tile / k.tiles_x, tx = tile - ty * k.tiles_x;
+    int ty = k.tiles_x == 1 ? tile : (int)__umulhi((unsigned)tile, k.tiles_x_magic), tx = tile - ty * k.tiles_x;
     ix = tx * kTile + (l & 7);
     iy = ty * kTile + (l >> 3);
     return q < k.padded_cells && ix < k.gx && iy < k.gy;
@@ -275,6 +279,12 @@ __device__ __forceinline__ int xcd_swizzle(int bid, int n_blocks) {
     int main = per * kXcd;
     if (bid >= main) return bid;
     return (bid % kXcd) * per + bid / kXcd;
+}
+
+// Batch element of a (renumbered) block of the cell-centric kernels.
+__device__ __forceinline__ int batch_of(const KParams &k, int bid) {
+    if (k.B == 1) return 0;
+    return k.bpb_magic ? (int)__umulhi((unsigned)bid, k.bpb_magic) : bid / k.blocks_per_batch;
 }
 
 __device__ __forceinline__ int replica_of(int ix, int iy) { return (ix + 5 * iy) & (kReplicas - 1); }

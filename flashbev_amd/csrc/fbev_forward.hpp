@@ -20,8 +20,8 @@ __device__ __forceinline__ LaneRole lane_role(const KParams &k, int lane) {
     // a lane group covers the channels of one cell; when long lists leave room for few slots,
     // several groups share a slot and take its entries in turn
     r.gps = k.groups_per_slot;
-    const int group = lane / k.lanes_per_slot;
-    r.slot = group / r.gps;
+    const int group = (int)(((unsigned)lane * k.lps_magic) >> 16);       // lane / lanes_per_slot
+    r.slot = (int)(((unsigned)group * k.gps_magic) >> 16);              // group / groups per slot
     r.sub = group - r.slot * r.gps;
     r.lis = lane - group * k.lanes_per_slot;
     r.carrier = r.slot < k.slots;
@@ -41,8 +41,9 @@ __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds 
     const float4 *lst = L.lst;
     const int gps = role.gps, slot = role.slot, sub = role.sub, lis = role.lis, span = role.span;
     const bool carrier = role.carrier;
-    constexpr int kUnitShift = VEC > 1 ? 4 : (sizeof(T) == 4 ? 2 : 1);
+    // a feature row starts at a 32-bit byte offset from the tensor's base: uniform base + 32-bit lane offset
     const char *fbytes = reinterpret_cast<const char *>(feats);
+    auto row_at = [&](unsigned byte_offset) { return reinterpret_cast<const T *>(fbytes + byte_offset); };
     {
         // phase A left the slot's cell in LDS: valid flag and ix | iy << 16
         const float4 mycell = L.cell[carrier ? slot : 0];
@@ -50,9 +51,10 @@ __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds 
         const bool mine = carrier && mycell.z != 0.0f;
         const int n = mine ? cnt[slot] : 0;
         const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * 2;
-        // the number of samples that enter the mean; the backward pass can reuse it
-        if (count_out != nullptr && mine && lis == 0 && sub == 0) count_out[((size_t)b * k.gy + iy) * k.gx + ix] = (float)n;
-        float *o = out + (((size_t)b * k.gy + iy) * k.gx + ix) * k.C;
+        // (the count: the number of samples that enter the mean; the backward pass can reuse it)
+        const unsigned cell_index = (unsigned)((b * k.gy + iy) * k.gx + ix);       // fits: the plan checks B * gy * gx
+        if (count_out != nullptr && mine && lis == 0 && sub == 0) count_out[cell_index] = (float)n;
+        float *o = out + (size_t)cell_index * k.C;
         for (int c0 = 0; out != nullptr && c0 < k.C; c0 += span) {
             float acc[CPL][VEC];
 #pragma unroll
@@ -63,19 +65,18 @@ __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds 
             auto gather = [&](int e) {
                 float4 w = my[2 * e];
                 float4 tf = my[2 * e + 1];
-                const T *p00 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.x) << kUnitShift));
-                const T *p01 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.y) << kUnitShift));
-                const T *p10 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.z) << kUnitShift));
-                const T *p11 = reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)__float_as_int(tf.w) << kUnitShift));
+                const unsigned o00 = (unsigned)__float_as_int(tf.x), o01 = (unsigned)__float_as_int(tf.y);
+                const unsigned o10 = (unsigned)__float_as_int(tf.z), o11 = (unsigned)__float_as_int(tf.w);
 #pragma unroll
                 for (int j = 0; j < CPL; ++j) {
                     int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
                     if (ch < k.C) {
+                        const unsigned chb = (unsigned)ch * (unsigned)sizeof(T);
                         float f00[VEC], f01[VEC], f10[VEC], f11[VEC];
-                        VecLoad<T, VEC>::ld(p00 + ch, f00);
-                        VecLoad<T, VEC>::ld(p01 + ch, f01);
-                        VecLoad<T, VEC>::ld(p10 + ch, f10);
-                        VecLoad<T, VEC>::ld(p11 + ch, f11);
+                        VecLoad<T, VEC>::ld(row_at(o00 + chb), f00);
+                        VecLoad<T, VEC>::ld(row_at(o01 + chb), f01);
+                        VecLoad<T, VEC>::ld(row_at(o10 + chb), f10);
+                        VecLoad<T, VEC>::ld(row_at(o11 + chb), f11);
 #pragma unroll
                         for (int v = 0; v < VEC; ++v) {
                             float a = acc[j][v];
@@ -93,6 +94,7 @@ __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds 
             // (group `sub` of the slot takes the entry pairs sub, sub + gps, ...)
             if (CPL == 1) {
                 const int ch = c0 + lis * VEC;
+                const unsigned chb = (unsigned)ch * (unsigned)sizeof(T);
                 int e = 2 * sub;
                 for (; ch < k.C && e + 1 < n; e += 2 * gps) {
                     const float4 wa = my[2 * e], ta = my[2 * e + 1], wb = my[2 * e + 2], tb = my[2 * e + 3];
@@ -102,7 +104,7 @@ __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds 
                     float f[8][VEC];
 #pragma unroll
                     for (int c = 0; c < 8; ++c)
-                        VecLoad<T, VEC>::ld(reinterpret_cast<const T *>(fbytes + ((size_t)(unsigned)off[c] << kUnitShift)) + ch, f[c]);
+                        VecLoad<T, VEC>::ld(row_at((unsigned)off[c] + chb), f[c]);
 #pragma unroll
                     for (int c = 0; c < 8; ++c)
 #pragma unroll
@@ -163,7 +165,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
-    const int b = bid / k.blocks_per_batch;
+    const int b = batch_of(k, bid);
     const int blk = bid - b * k.blocks_per_batch;
 
     const WaveLds L = block_lds_setup(k, smem, proj, b, 2);
@@ -279,7 +281,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_cached_ker
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
-    const int b = bid / k.blocks_per_batch;
+    const int b = batch_of(k, bid);
     const int blk = bid - b * k.blocks_per_batch;
     const WaveLds L = wave_lds_view(k, smem, 2);
     const LaneRole role = lane_role<VEC, CPL>(k, lane);
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_geometry_cache_ker
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int bid = xcd_swizzle(blockIdx.x, k.n_blocks);
-    const int b = bid / k.blocks_per_batch;
+    const int b = batch_of(k, bid);
     const int blk = bid - b * k.blocks_per_batch;
     const WaveLds L = block_lds_setup(k, smem, proj, b, 1);
     int *counts = reinterpret_cast<int *>(static_cast<char *>(cache) + kCacheHeaderBytes);

@@ -118,10 +118,17 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     const int full_vec = 16 / es;
     plan->vec = (allow_vec && k.C % full_vec == 0) ? full_vec : 1;
     {
-        // feature rows are addressed in 32-bit units (16 bytes, or one element off the vector paths)
-        const long long units = plan->vec > 1 ? (long long)k.C * es / 16 : k.C;
-        if ((long long)k.B * k.N * k.H * k.W * units >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
-        k.row_units = (int)units;
+        // feature rows are addressed by 32-bit byte offsets from the tensor's base (the gather loops then
+        // form an address with one 32-bit add): the feature tensor stays below 4 GiB
+        if ((long long)k.B * k.N * k.H * k.W * k.C * es >= (1ll << 32)) return FBEV_ERR_TOO_LARGE;
+        k.row_units = k.C * es;
+        // exact division of a tile index by tiles_x: umulhi(tile, ceil(2^32 / tiles_x)) is the quotient for
+        // every tile with tile * tiles_x < 2^32
+        const long long tiles = (long long)k.tiles_x * k.tiles_y;
+        if (tiles * k.tiles_x >= (1ll << 32)) return FBEV_ERR_TOO_LARGE;
+        // (a divisor of 1 has no 32-bit magic; the kernels test for it)
+        k.tiles_x_magic = k.tiles_x > 1 ? (unsigned)(((1ull << 32) + k.tiles_x - 1) / k.tiles_x) : 0u;
+        k.cams_magic = k.N > 1 ? (unsigned)(((1ull << 32) + k.N - 1) / k.N) : 0u;
     }
     const int cq = (k.C + plan->vec - 1) / plan->vec;      // channel vectors per texel
     int lps = cq < kWave ? cq : kWave;
@@ -143,6 +150,8 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     }
     k.slots = slots;
     k.groups_per_slot = (kWave / lps) / slots;     // >= 1: slots <= kWave / lps
+    k.lps_magic = 65535u / (unsigned)lps + 1u;
+    k.gps_magic = 65535u / (unsigned)k.groups_per_slot + 1u;
     k.list_cap = k.NZ;
     // enough wavefronts to fill 256 CUs several times over before a wavefront takes more rounds,
     // and never many rounds: cells differ widely in their number of samples, and short wavefronts
@@ -155,6 +164,9 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     const int cells_per_block = waves * k.slots * k.rounds;
     k.blocks_per_batch = (k.padded_cells + cells_per_block - 1) / cells_per_block;
     k.n_blocks = k.blocks_per_batch * k.B;
+    // exact for every block index when n_blocks * blocks_per_batch < 2^32; otherwise the kernels divide
+    k.bpb_magic = (k.blocks_per_batch > 1 && (long long)k.n_blocks * k.blocks_per_batch < (1ll << 32))
+                      ? (unsigned)(((1ull << 32) + k.blocks_per_batch - 1) / k.blocks_per_batch) : 0u;
     const size_t p_f4 = (size_t)(k.N * 12 + 3) / 4;
     const size_t cols = (size_t)k.slots * k.N, dec_f4 = (cols + 3) / 4;
     const size_t cand_f4 = ((size_t)k.slots * k.NZ + 3) / 4, z_f4 = ((size_t)k.gz + 3) / 4;

@@ -62,7 +62,7 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
     for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
         Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
-        const int slot = i / k.N, cam = i - slot * k.N;
+        const int slot = k.N == 1 ? i : (int)__umulhi((unsigned)i, k.cams_magic), cam = i - slot * k.N;
         dec[i] = (slot << 28) | (cam << 16);
     }
     for (int i = threadIdx.x; i < k.gz; i += blockDim.x) zt[i] = voxel_coord(k.zmin, i, k.vz);
@@ -73,7 +73,7 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 // Entry of a compacted list: ENTRY_F4 float4 words.
 //   forward   word 0: corner weights already multiplied by the depth weight
 //             word 1: where the four texels' feature rows start, in address units (texel index
-//                     ((b*N+n)*H + v)*W + u times KParams::row_units) as int bits (t00, t01, t10, t11):
+//                     ((b*N+n)*H + v)*W + u times KParams::row_units) as unsigned bits (t00, t01, t10, t11):
 //                     the gather loop then forms an address with one shift-add, not a 64-bit multiply
 //   cache     one word: du, dv, t00 << 2 | (u1 != u0) | (v1 != v0) << 1, depth along the optical axis
 //   backward  word 0: du, dv, t00, (u1 != u0) | (v1 != v0) << 1 -- the four weights and texels
