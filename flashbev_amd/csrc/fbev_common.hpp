@@ -193,6 +193,32 @@ __device__ __forceinline__ Geom project_column(const KParams &k, const float *P,
     return g;
 }
 
+// The same sample, evaluated without branches (the sample phase runs it on lanes that passed a cheap
+// test, nearly all of which are in view): every operation is the one project_column performs, in the
+// same order, so a sample in view gets the same bits; a sample out of view gets clamped indices and
+// fractions nobody uses.
+__device__ __forceinline__ Geom project_column_flat(const KParams &k, const float *P, float au, float av, float ad, float z) {
+    Geom g;
+    const float U = (au + P[2] * z) + P[3];
+    const float V = (av + P[6] * z) + P[7];
+    const float D = (ad + P[10] * z) + P[11];
+    g.depth = D;
+    const float dc = fmaxf(D, k.eps);
+    const float ui = U / dc;
+    const float vi = V / dc;
+    const float fu = (ui / k.Wi_f) * k.W_f;
+    const float fv = (vi / k.Hi_f) * k.H_f;
+    g.valid = D > 0.0f && fu >= 0.0f && fu < k.W_f && fv >= 0.0f && fv < k.H_f;
+    const float u0f = floorf(fu), v0f = floorf(fv);
+    g.du = fu - u0f;
+    g.dv = fv - v0f;
+    g.u0 = min(max((int)u0f, 0), k.W - 1);
+    g.u1 = min(g.u0 + 1, k.W - 1);
+    g.v0 = min(max((int)v0f, 0), k.H - 1);
+    g.v1 = min(g.v0 + 1, k.H - 1);
+    return g;
+}
+
 __device__ __forceinline__ Geom project_sample(const KParams &k, const float *P, float x, float y, float z) {
     return project_column(k, P, P[0] * x + P[1] * y, P[4] * x + P[5] * y, P[8] * x + P[9] * y, z);
 }

@@ -198,38 +198,39 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         if (active) {
             const float4 c = L.cell[slot];
             cellxy = __float_as_int(c.w);
-            Geom g = project_column(k, L.Pm + cam * 12, col.x, col.y, col.z, L.zt[key & 0xffffu]);
-            if (g.valid) {
-                float w00 = (1.0f - g.du) * (1.0f - g.dv);
-                float w01 = (1.0f - g.du) * g.dv;
-                float w10 = g.du * (1.0f - g.dv);
-                float w11 = g.du * g.dv;
-                int rowbase = (b * k.N + cam) * k.H;
-                int t00 = (rowbase + g.v0) * k.W + g.u0;
-                int t01 = (rowbase + g.v1) * k.W + g.u0;
-                int t10 = (rowbase + g.v0) * k.W + g.u1;
-                int t11 = (rowbase + g.v1) * k.W + g.u1;
-                DepthEval e;
-                if (MODE == kModeCache) {
-                    e.keep = true;       // every sample in view is listed; the depth model comes later
-                    e.wgt = e.a = e.b = 0.0f;
-                    e.k0 = e.k1 = 0;
-                } else {
-                    e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
-                }
-                keep = e.keep;
-                tx = make_int4(t00, t01, t10, t11);
-                if (MODE == kModeCache) {
-                    const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
-                    w0 = make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), g.depth);
-                } else if (BACKWARD) {
-                    const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
-                    w0 = FILLING ? make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1))
-                                           : make_float4(g.du, g.dv, __int_as_float(t00), __int_as_float(fl));
-                    w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
-                } else {
-                    w0 = make_float4(w00 * e.wgt, w01 * e.wgt, w10 * e.wgt, w11 * e.wgt);
-                }
+            // no branch on the outcome of the exact test: nearly every candidate passes it, and the joins
+            // of a branch here cost more moves than the arithmetic it skips (indices are clamped, so the
+            // depth loads of a sample out of view read valid memory and their result is dropped)
+            const Geom g = project_column_flat(k, L.Pm + cam * 12, col.x, col.y, col.z, L.zt[key & 0xffffu]);
+            const float w00 = (1.0f - g.du) * (1.0f - g.dv);
+            const float w01 = (1.0f - g.du) * g.dv;
+            const float w10 = g.du * (1.0f - g.dv);
+            const float w11 = g.du * g.dv;
+            const int rowbase = (b * k.N + cam) * k.H;
+            const int t00 = (rowbase + g.v0) * k.W + g.u0;
+            const int t01 = (rowbase + g.v1) * k.W + g.u0;
+            const int t10 = (rowbase + g.v0) * k.W + g.u1;
+            const int t11 = (rowbase + g.v1) * k.W + g.u1;
+            DepthEval e;
+            if (MODE == kModeCache) {
+                e.keep = true;       // every sample in view is listed; the depth model comes later
+                e.wgt = e.a = e.b = 0.0f;
+                e.k0 = e.k1 = 0;
+            } else {
+                e = eval_depth<T>(k, depth, t00, t01, t10, t11, w00, w01, w10, w11, g.depth);
+            }
+            keep = g.valid && e.keep;
+            tx = make_int4(t00, t01, t10, t11);
+            if (MODE == kModeCache) {
+                const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
+                w0 = make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), g.depth);
+            } else if (BACKWARD) {
+                const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
+                w0 = FILLING ? make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1))
+                                       : make_float4(g.du, g.dv, __int_as_float(t00), __int_as_float(fl));
+                w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
+            } else {
+                w0 = make_float4(w00 * e.wgt, w01 * e.wgt, w10 * e.wgt, w11 * e.wgt);
             }
         }
         const int prev_slot = __shfl_up(slot, 1, kWave);
