@@ -93,13 +93,20 @@ class Runner:
                     x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
                     x["image_size"], x["grid_size"], self.dist)
 
-    def forward(self):
+    def forward(self, cache=None):
         x, w = self.x, self.w
         self.ext.flash_bevpool_forward(
             x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"], x["image_size"],
             x["grid_size"], self.vsize[0], self.vsize[1], self.vsize[2], self.vmin[0], self.vmin[1],
             self.vmin[2], self.out, self.out.numel(), self.dist, True, True, False, False, self.eps, self.thr,
-            w.depth_range[0], w.depth_range[1], 0, self.counts)
+            w.depth_range[0], w.depth_range[1], 0, self.counts, cache)
+
+    def geometry_cache(self):
+        """Per-cell lists of the samples in view for this calibration and grid (built once)."""
+        x, w = self.x, self.w
+        H, W = w.feat_hw
+        return self.ext.build_geometry_cache(x["projection_matrices"], H, W, w.image_hw[0], w.image_hw[1],
+                                             list(w.grid_size), self.vmin, self.vsize, self.eps)
 
     def backward(self):
         x, w = self.x, self.w
@@ -140,6 +147,28 @@ def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
     fwd = [ev[i][0].elapsed_time(ev[i][1]) for i in range(steps)]
     bwd = [ev[i][2].elapsed_time(ev[i][3]) for i in range(steps)] if with_backward else []
     return (t1 - t0) * 1e3 / steps, fwd, bwd
+
+
+def time_cached_forward(r: Runner, steps: int, warmup: int):
+    """Forward on cached geometry (the lists of samples in view built once, outside the timed region:
+    what a fixed rig at inference allows); checked against the plain forward, bit for bit, first."""
+    r.forward()
+    want = r.out.clone()
+    cache = r.geometry_cache()
+    r.out.zero_()
+    r.forward(cache)
+    torch.cuda.synchronize()
+    if not torch.equal(r.out, want):
+        raise RuntimeError("forward on cached geometry differs from the forward")
+    for _ in range(warmup):
+        r.forward(cache)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in ev:
+        a.record()
+        r.forward(cache)
+        b.record()
+    torch.cuda.synchronize()
+    return statistics.mean(a.elapsed_time(b) for a, b in ev), cache.numel()
 
 
 def time_graph_steps(r: Runner, steps: int, warmup: int):
@@ -215,6 +244,20 @@ def time_operator_steps(r: Runner, steps: int, warmup: int):
             torch.cuda.synchronize()
             chunks.append((time.perf_counter() - t0) * 1e3 / max(1, steps // 5))
         got[name] = statistics.median(chunks)
+        if name == "fwd_bwd":
+            # the same with the autograd engine on the calling thread (no hand-over to its device thread)
+            with torch.autograd.set_multithreading_enabled(False):
+                for _ in range(10):
+                    step()
+                torch.cuda.synchronize()
+                chunks = []
+                for _ in range(5):
+                    t0 = time.perf_counter()
+                    for _ in range(max(1, steps // 5)):
+                        step()
+                    torch.cuda.synchronize()
+                    chunks.append((time.perf_counter() - t0) * 1e3 / max(1, steps // 5))
+            got["fwd_bwd_engine_on_calling_thread"] = statistics.median(chunks)
     return got
 
 
@@ -277,6 +320,8 @@ def other_workloads(steps: int, warmup: int, backward_mode: int):
                                "frac_hbm": bb / b_ms / 1e6 / HBM_PEAK_GBS}
             rec["ms_per_step_fwd_bwd"] = ms
             rec["frac_hbm_fwd_bwd"] = (fb + bb) / ms / 1e6 / HBM_PEAK_GBS
+        c_ms, c_bytes = time_cached_forward(r, steps, warmup)
+        rec["forward_cached_geometry"] = {"ms": c_ms, "frac_hbm": fb / c_ms / 1e6 / HBM_PEAK_GBS, "cache_bytes": c_bytes}
         rec["kept_samples"] = int(r.counts.sum().item())
         got[name] = rec
         del r
@@ -339,6 +384,9 @@ def main():
     ap.add_argument("--table", action="store_true")
     ap.add_argument("--table-dir", default="bench_out", help="directory (under the repository) for the --table files")
     ap.add_argument("--no-graph", action="store_true", help="time eagerly queued steps only")
+    ap.add_argument("--only-steps", nargs="?", const="plain", default=None, choices=("plain", "cached"),
+                    help="run only warm-up and timed steps of the workload (for profilers); 'cached': forward on "
+                         "cached geometry")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the two large configurations otherwise timed beside the default workload")
     ap.add_argument("--backward-mode", type=int, default=0, choices=(0, 1, 2, 3),
@@ -366,6 +414,21 @@ def main():
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n}))
         return
     r = Runner(w, args.depth, backward_mode=args.backward_mode)
+    if args.only_steps:
+        # for profilers: nothing but warm-up and timed steps of the one workload (every launch of the run
+        # belongs to it), optionally with the forward on cached geometry in place of the forward
+        cache = r.geometry_cache() if args.only_steps == "cached" else None
+        for _ in range(args.warmup):
+            r.forward(cache); r.backward()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            r.forward(cache); r.backward()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        print(json.dumps({"workload": w.name, "depth_model": args.depth, "steps": args.steps, "warmup": args.warmup,
+                          "ms_per_step": ms, "kept_samples": int(r.counts.sum().item())}), flush=True)
+        return
     eager_ms, fwd, bwd = time_steps(r, args.steps, args.warmup, True)
     graph_ms = None if args.no_graph else time_graph_steps(r, args.steps, args.warmup)
     ms = eager_ms
@@ -376,6 +439,7 @@ def main():
     del r0
     kernels = profile_steps(r, args.steps)
     op_ms = time_operator_steps(r, args.steps, args.warmup)
+    cached_ms, cache_bytes = time_cached_forward(r, args.steps, args.warmup)
     fwd_ms, bwd_ms = statistics.mean(fwd), statistics.mean(bwd)
     kept = int(r.counts.sum().item())          # samples that passed the view and weight tests
     es = 4 if w.dtype == torch.float32 else 2
@@ -403,7 +467,9 @@ def main():
         "ms_per_step_eager": eager_ms, "ms_per_step_graph": graph_ms, "ms_per_step_per_call_workspace": percall_ms,
         "fwd_call_ms": stats(fwd), "bwd_call_ms": stats(bwd),
         # the same work through the autograd operator, output and gradient allocation included
-        "operator_ms_incl_alloc": {"fwd": op_ms["fwd"], "fwd_bwd": op_ms["fwd_bwd"]},
+        "operator_ms_incl_alloc": op_ms,
+        # forward on cached geometry (fixed calibration): event-timed call, cache size in bytes
+        "fwd_cached_geometry": {"call_ms": cached_ms, "cache_bytes": cache_bytes},
         # not HBM traffic: what the gathers request from the caches (every kept sample reads four
         # feature rows and eight depth values forward, and the same rows plus its cell's
         # grad_out row backward) -- the figure a latency/L2-bound pass is better judged by
