@@ -67,6 +67,11 @@ def _pair_capacity(batch: int, cams: int, grid) -> int:
 _workspaces: "collections.OrderedDict" = collections.OrderedDict()
 
 
+def release_workspaces() -> None:
+    """Drop the persistent backward workspaces kept so far (they are prepared again on demand)."""
+    _workspaces.clear()
+
+
 def _stream_id(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 

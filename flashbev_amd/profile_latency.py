@@ -31,7 +31,7 @@ from typing import Dict, List, Optional
 import numpy as np
 import torch
 
-from .flash_bevpool import flash_bevpool
+from .flash_bevpool import flash_bevpool, release_workspaces
 from .rig import load_calibration_params, rig_projection, surround_rig
 from .sampling_vt import SamplingVT
 from .workloads import SURROUND_YAWS
@@ -126,6 +126,7 @@ def time_calls(fn, num_warmup: int, num_iterations: int) -> Dict[str, float]:
 
 
 def run_point(args: argparse.Namespace, num_bins: int, num_cams: int, threshold: float) -> List[Dict]:
+    release_workspaces()      # the previous point's backward workspaces are not this point's memory
     grid = grid_for(args, num_bins)
     sizes = [int(round((grid[a][1] - grid[a][0]) / grid[a][2])) for a in "xyz"]
     roi = [grid["x"][0], grid["x"][1], grid["y"][0], grid["y"][1], grid["z"][0], grid["z"][1]]
