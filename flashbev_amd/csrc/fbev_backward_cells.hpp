@@ -71,11 +71,12 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_count_kernel(KPara
     const int b = batch_of(k, bid);
     const int blk = bid - b * k.blocks_per_batch;
     const WaveLds L = block_lds_setup(k, smem, proj, b, 0);
-    const int cells_per_wave = k.slots * k.rounds;
+    const int cells_per_wave = k.slots_a * k.rounds;
     for (int r = 0; r < k.rounds; ++r) {
-        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
+        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots_a;
         if (q0 >= k.padded_cells) break;
-        phase_a<0, T, kModeCount>(k, L, depth, b, q0, lane, nullptr, counts, 0);
+        const int n_cand = phase_a_candidates<false>(k, L, q0, lane);     // group boundaries are not needed
+        phase_a_samples<0, T, kModeCount>(k, L, depth, b, lane, 0, n_cand, nullptr, counts, 0);      // no entries: no pool
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(1024) void fbev_scan_sums_kernel(int *v, int n) {
 // map); FILL = 2: the same with one claim per run of samples on one texel.
 // `cursor` holds, on entry, the start (within its scan chunk) of every (texel, replica)
 // segment; phase A advances it, so on exit cursor[i] is the END of segment i.
-template <typename T, int VEC, int CPL, int FILL>
+template <typename T, int VEC, int CPL, int FILL, bool BATCHED>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_kernel(
     KParams k, const float *__restrict__ grad_out, const T *__restrict__ depth, const T *__restrict__ feats,
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     lds_counter *cnt = L.cnt;
     float4 *lst = L.lst;
 
-    const int cells_per_wave = k.slots * k.rounds;
+    const int cells_per_wave = k.slots_a * k.rounds;
     // lane groups of lanes_per_slot lanes; the groups_per_slot groups of a slot take its entries in turn
     const int gps = k.groups_per_slot;
     const int group = (int)(((unsigned)lane * k.lps_magic) >> 16);       // lane / lanes_per_slot
@@ -214,14 +215,21 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     const unsigned row_step_v = (unsigned)(k.W * k.row_units);      // one feature-map row down
 
     for (int r = 0; r < k.rounds; ++r) {
-        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
+        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots_a;
         if (q0 >= k.padded_cells) break;
-        int ix = 0, iy = 0;
-        const bool mine = carrier && cell_of(k, q0 + slot, ix, iy);
-        const int cell = (b * k.gy + iy) * k.gx + ix;
-        const float *go = grad_out + (size_t)cell * k.C;
-        // the cell's grad_out row (first channel pass) is requested before phase A and arrives
-        // while the samples are evaluated
+        // the lane's cell in the group of the batch it is working on
+        bool mine = false;
+        int cell = 0;
+        const float *go = grad_out;
+        auto enter_group = [&](int j) {
+            int ix = 0, iy = 0;
+            mine = carrier && cell_of(k, q0 + j * k.slots + slot, ix, iy);
+            cell = (b * k.gy + iy) * k.gx + ix;
+            go = grad_out + (size_t)cell * k.C;
+        };
+        // the grad_out row of the cell (first channel pass) of the first group that goes through stage 2
+        // is requested before the sample phase and arrives while the samples are evaluated; the
+        // groups behind it in a batch ask for theirs when their turn comes
         float g[CPL][VEC];
         auto load_g = [&](int c0) {
 #pragma unroll
@@ -242,18 +250,36 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 }
             }
         };
+        enter_group(0);
         load_g(0);
-        phase_a<EF4, T, FILL == 2 ? kModeFillRuns : (FILL ? kModeFill : kModeScatter)>(k, L, depth, b, q0, lane, chunk_prefix, cursor, pair_cap);
+        const int n_cand = phase_a_candidates<BATCHED>(k, L, q0, lane);
+        // all groups of the batch through stage 2 together when the pool is sure to hold what they keep
+        const int n_groups = BATCHED ? k.batch_groups : 1;
+        const int step = n_cand <= k.pool_cap ? n_groups : 1;
+        for (int g0 = 0; g0 < n_groups; g0 += step) {
+        if (BATCHED && g0 > 0) {
+            enter_group(g0);
+            load_g(0);
+        }
+        phase_a_samples<EF4, T, FILL == 2 ? kModeFillRuns : (FILL ? kModeFill : kModeScatter)>(
+            k, L, depth, b, lane, BATCHED ? L.gcand[g0] : 0, BATCHED ? L.gcand[g0 + step] : n_cand, chunk_prefix, cursor,
+            pair_cap);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        for (int grp = g0; grp < g0 + step; ++grp) {
+        if (BATCHED && grp > g0) {
+            enter_group(grp);
+            load_g(0);
+        }
+        const int slot_a = carrier ? grp * k.slots + slot : 0;
 
-        const int n = mine ? cnt[slot] : 0;
+        const int n = mine ? cnt[slot_a] : 0;
         // every lane of the wavefront takes part in the shuffles below, so all lanes run
         // the longest list of the wavefront and idle past their own.
         int n_max = n;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) n_max = max(n_max, __shfl_xor(n_max, off, kWave));
-        float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * EF4;
+        float4 *my = lst + (size_t)L.start[slot_a] * EF4;
         const float inv = (k.reduce_sum || n == 0) ? 1.0f : 1.0f / (float)n;
 
         for (int c0 = 0; c0 < k.C; c0 += span) {
@@ -413,7 +439,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 }
             }
         }
+        }      // the groups of this pass through stage 2
         __builtin_amdgcn_wave_barrier();
+        }      // the passes of the batch through stage 2
     }
 }
 

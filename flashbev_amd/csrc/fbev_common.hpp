@@ -80,8 +80,11 @@ struct KParams {
     int tiles_x, tiles_y;
     int padded_cells;    // tiles_x * tiles_y * 64
     int blocks_per_batch;
-    int slots;           // S: cells per wavefront per round
-    int rounds;          // rounds per wavefront
+    int slots;           // S: cells per group (phase B works on one group: its lane groups cover S cells)
+    int batch_groups;    // groups that go through the sample phase together (1 to 4)
+    int slots_a;         // cells per batch = slots * batch_groups (at most 16)
+    int pool_cap;        // entries the pool of a wavefront holds (= slots * NZ)
+    int rounds;          // batches per wavefront
     int lanes_per_slot;  // lanes that carry channels in phase B (one lane group)
     int groups_per_slot; // lane groups that share a slot's list (more than one when long lists leave few slots)
     int list_cap;        // entries per slot list (= NZ)

@@ -29,28 +29,30 @@ __device__ __forceinline__ LaneRole lane_role(const KParams &k, int lane) {
     return r;
 }
 
-// Phase B of one round: every slot walks its list of kept samples (phase A left the lists, their
-// lengths and the cells in LDS) and stores its cell's row of the output.
+// Phase B of one group of a batch: every slot walks its cell's list of kept samples (the sample phase
+// left the entries, where each cell's start, their number and the cells in LDS) and stores its
+// cell's row of the output.
 // STREAM: the output is stored with non-temporal stores (a template parameter: as a run-time
 // choice between two stores the compiler merges them into one ordinary store).
 template <typename T, int VEC, int CPL, bool STREAM>
 __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds &L, const LaneRole &role, int b,
-                                                const T *__restrict__ feats, float *__restrict__ out,
+                                                int group, const T *__restrict__ feats, float *__restrict__ out,
                                                 float *__restrict__ count_out) {
     lds_counter *cnt = L.cnt;
     const float4 *lst = L.lst;
-    const int gps = role.gps, slot = role.slot, sub = role.sub, lis = role.lis, span = role.span;
+    const int gps = role.gps, sub = role.sub, lis = role.lis, span = role.span;
     const bool carrier = role.carrier;
+    const int slot = carrier ? group * k.slots + role.slot : 0;      // the lane's cell within the batch
     // a feature row starts at a 32-bit byte offset from the tensor's base: uniform base + 32-bit lane offset
     const char *fbytes = reinterpret_cast<const char *>(feats);
     auto row_at = [&](unsigned byte_offset) { return reinterpret_cast<const T *>(fbytes + byte_offset); };
     {
         // phase A left the slot's cell in LDS: valid flag and ix | iy << 16
-        const float4 mycell = L.cell[carrier ? slot : 0];
+        const float4 mycell = L.cell[slot];
         const int ix = __float_as_int(mycell.w) & 0xffff, iy = __float_as_int(mycell.w) >> 16;
         const bool mine = carrier && mycell.z != 0.0f;
         const int n = mine ? cnt[slot] : 0;
-        const float4 *my = lst + (size_t)(carrier ? slot : 0) * k.list_cap * 2;
+        const float4 *my = lst + (size_t)L.start[slot] * 2;
         // (the count: the number of samples that enter the mean; the backward pass can reuse it)
         const unsigned cell_index = (unsigned)((b * k.gy + iy) * k.gx + ix);       // fits: the plan checks B * gy * gx
         if (count_out != nullptr && mine && lis == 0 && sub == 0) count_out[cell_index] = (float)n;
@@ -157,7 +159,7 @@ __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds 
     }
 }
 
-template <typename T, int VEC, int CPL, bool STREAM>
+template <typename T, int VEC, int CPL, bool STREAM, bool BATCHED>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     KParams k, const T *__restrict__ depth, const T *__restrict__ feats, const float *__restrict__ proj,
     float *__restrict__ out, float *__restrict__ count_out) {
@@ -170,15 +172,22 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
 
     const WaveLds L = block_lds_setup(k, smem, proj, b, 2);
     const LaneRole role = lane_role<VEC, CPL>(k, lane);
-    const int cells_per_wave = k.slots * k.rounds;
+    const int cells_per_wave = k.slots_a * k.rounds;
     for (int r = 0; r < k.rounds; ++r) {
-        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
+        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots_a;
         if (q0 >= k.padded_cells) break;
-        phase_a<2, T, kModeForward>(k, L, depth, b, q0, lane);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        forward_phase_b<T, VEC, CPL, STREAM>(k, L, role, b, feats, out, count_out);
-        __builtin_amdgcn_wave_barrier();
+        const int n_cand = phase_a_candidates<BATCHED>(k, L, q0, lane);
+        // all groups of the batch through stage 2 together when the pool is sure to hold what they keep
+        const int n_groups = BATCHED ? k.batch_groups : 1;
+        const int step = n_cand <= k.pool_cap ? n_groups : 1;
+        for (int g = 0; g < n_groups; g += step) {
+            phase_a_samples<2, T, kModeForward>(k, L, depth, b, lane, BATCHED ? L.gcand[g] : 0,
+                                                BATCHED ? L.gcand[g + step] : n_cand);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            for (int j = g; j < g + step; ++j) forward_phase_b<T, VEC, CPL, STREAM>(k, L, role, b, j, feats, out, count_out);
+            __builtin_amdgcn_wave_barrier();
+        }
     }
 }
 
@@ -207,7 +216,10 @@ template <typename T>
 __device__ __forceinline__ void phase_a_cached(const KParams &k, const WaveLds &L, const T *__restrict__ depth,
                                                const int *__restrict__ counts, const float4 *__restrict__ entries,
                                                int b, int q0, int lane) {
-    if (lane < 16) L.cnt[lane] = 0;
+    if (lane < k.slots) {
+        L.cnt[lane] = 0;
+        L.start[lane] = lane * k.NZ;      // a cell's entries start at its own stretch of the pool here
+    }
     // lane s < slots: its cell, the number of cached samples, and where they start among the round's
     int mine_n = 0;
     if (lane < k.slots) {
@@ -264,7 +276,7 @@ __device__ __forceinline__ void phase_a_cached(const KParams &k, const WaveLds &
         const int prefix = __popcll(m & seg & lanemask_lt(lane));
         const int old = active ? L.cnt[slot] : 0;
         if (keep) {
-            float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * 2;
+            float4 *e = L.lst + (size_t)(slot * k.NZ + old + prefix) * 2;
             e[0] = w0;
             e[1] = make_float4(__int_as_float(tx.x * k.row_units), __int_as_float(tx.y * k.row_units),
                                __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
@@ -288,14 +300,16 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_cached_ker
     const int *counts = cache_counts(cache);
     const float4 *entries = reinterpret_cast<const float4 *>(static_cast<const char *>(cache) +
                                                              cache_entries_offset((long long)k.B * k.padded_cells));
-    const int cells_per_wave = k.slots * k.rounds;
-    for (int r = 0; r < k.rounds; ++r) {
+    // (the cached lists are walked one group of `slots` cells at a time: their lengths are known, and
+    // each cell's entries go to its own stretch of the pool)
+    const int cells_per_wave = k.slots_a * k.rounds;
+    for (int r = 0; r < k.rounds * k.batch_groups; ++r) {
         const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
         phase_a_cached<T>(k, L, depth, counts, entries, b, q0, lane);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        forward_phase_b<T, VEC, CPL, STREAM>(k, L, role, b, feats, out, count_out);
+        forward_phase_b<T, VEC, CPL, STREAM>(k, L, role, b, 0, feats, out, count_out);
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -320,20 +334,24 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_geometry_cache_ker
     }
     float4 *entries = reinterpret_cast<float4 *>(static_cast<char *>(cache) +
                                                  cache_entries_offset((long long)k.B * k.padded_cells));
-    const int cells_per_wave = k.slots * k.rounds;
+    const int cells_per_wave = k.slots_a * k.rounds;
     for (int r = 0; r < k.rounds; ++r) {
-        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
+        const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots_a;
         if (q0 >= k.padded_cells) break;
-        phase_a<1, float, kModeCache>(k, L, nullptr, b, q0, lane);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        for (int s = 0; s < k.slots && q0 + s < k.padded_cells; ++s) {
-            const size_t cell = (size_t)b * k.padded_cells + q0 + s;
-            const int n = L.cnt[s];
-            if (lane == 0) counts[cell] = n;
-            for (int i = lane; i < n; i += kWave) entries[cell * k.NZ + i] = L.lst[(size_t)s * k.list_cap + i];
+        const int n_cand = phase_a_candidates<true>(k, L, q0, lane);
+        const int step = n_cand <= k.pool_cap ? k.batch_groups : 1;
+        for (int g = 0; g < k.batch_groups; g += step) {
+            phase_a_samples<1, float, kModeCache>(k, L, nullptr, b, lane, L.gcand[g], L.gcand[g + step]);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            for (int s = g * k.slots; s < (g + step) * k.slots && q0 + s < k.padded_cells; ++s) {
+                const size_t cell = (size_t)b * k.padded_cells + q0 + s;
+                const int n = L.cnt[s], first = L.start[s];
+                if (lane == 0) counts[cell] = n;
+                for (int i = lane; i < n; i += kWave) entries[cell * k.NZ + i] = L.lst[first + i];
+            }
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_wave_barrier();
     }
 }
 

@@ -35,6 +35,7 @@
 
 #include <atomic>
 #include <mutex>
+#include <type_traits>
 #include <vector>
 
 #include "flashbev_hip.h"
@@ -89,7 +90,7 @@ int validate(const fbev_problem *p, bool need_channels) {
 }
 
 int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWavesPerBlock, int max_rounds = 3,
-              int slot_budget = kMaxSlotLdsBytes) {
+              int slot_budget = kMaxSlotLdsBytes, int max_batch = 4) {
     const int entry_bytes = 32 + 4;      // an entry (two float4 in every kernel) and its candidate index
     KParams &k = plan->k;
     k.B = p->batch; k.N = p->num_cams; k.H = p->feat_h; k.W = p->feat_w; k.C = p->channels;
@@ -153,30 +154,48 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     k.lps_magic = 65535u / (unsigned)lps + 1u;
     k.gps_magic = 65535u / (unsigned)k.groups_per_slot + 1u;
     k.list_cap = k.NZ;
+    k.pool_cap = slots * k.NZ;       // what one group of `slots` cells can keep at most
     // enough wavefronts to fill 256 CUs several times over before a wavefront takes more rounds,
     // and never many rounds: cells differ widely in their number of samples, and short wavefronts
     // even that out (training-size cell pass: 439 / 406 / 399 / 404 / 439 us with at most
     // 8 / 4 / 3 / 2 / 1 rounds; the forward does not care)
     const long long groups = ((long long)k.padded_cells + slots - 1) / slots * k.B;
     int rounds = (int)(groups / (256ll * 4 * 8 * 2));
-    k.rounds = rounds < 1 ? 1 : (rounds > max_rounds ? max_rounds : rounds);
+    rounds = rounds < 1 ? 1 : (rounds > max_rounds ? max_rounds : rounds);
+    // Groups of one batch: the sample phase runs over `batch` groups of `slots` cells together, so that
+    // its 64-lane passes are filled (about one sample in six is in view: a group with fewer than some
+    // forty in-view samples leaves stage 2 half empty).  Never more groups than the wavefront has rounds
+    // (a small problem keeps its many short wavefronts), at most four, at most 16 cells.
+    int batch = 1;
+    if (max_batch > 1 && plan->vec > 1) {
+        const int expect = (slots * k.NZ + 5) / 6;          // candidates of one group, roughly
+        batch = expect > 0 ? (64 + expect / 2) / expect : 1;      // as many groups as fill one pass, rounded
+        if (batch > max_batch) batch = max_batch;
+        if (batch > rounds) batch = rounds;
+        while (batch > 1 && (slots * batch > 16 || (long long)slots * batch * k.NZ >= 4096)) --batch;
+        if (batch < 1) batch = 1;
+    }
+    k.batch_groups = batch;
+    k.slots_a = slots * batch;
+    k.rounds = (rounds + batch - 1) / batch;          // batches per wavefront
     k.waves = waves;
-    const int cells_per_block = waves * k.slots * k.rounds;
+    const int cells_per_block = waves * k.slots_a * k.rounds;
     k.blocks_per_batch = (k.padded_cells + cells_per_block - 1) / cells_per_block;
     k.n_blocks = k.blocks_per_batch * k.B;
     // exact for every block index when n_blocks * blocks_per_batch < 2^32; otherwise the kernels divide
     k.bpb_magic = (k.blocks_per_batch > 1 && (long long)k.n_blocks * k.blocks_per_batch < (1ll << 32))
                       ? (unsigned)(((1ull << 32) + k.blocks_per_batch - 1) / k.blocks_per_batch) : 0u;
     const size_t p_f4 = (size_t)(k.N * 12 + 3) / 4;
-    const size_t cols = (size_t)k.slots * k.N, dec_f4 = (cols + 3) / 4;
-    const size_t cand_f4 = ((size_t)k.slots * k.NZ + 3) / 4, z_f4 = ((size_t)k.gz + 3) / 4;
+    const size_t cols = (size_t)k.slots_a * k.N, dec_f4 = (cols + 3) / 4;
+    const size_t cand_f4 = ((size_t)k.slots_a * k.NZ + 3) / 4, z_f4 = ((size_t)k.gz + 3) / 4;
     auto block_lds = [&](int entry_f4) {
         return (p_f4 + dec_f4 + z_f4 +
-                (size_t)waves * (20 + cols + dec_f4 + cand_f4 + (size_t)k.slots * k.list_cap * entry_f4)) * 16;
+                (size_t)waves * ((2 * (size_t)k.slots_a + 8 + 3) / 4 + k.slots_a + cols + dec_f4 + cand_f4 +
+                                 (size_t)k.pool_cap * entry_f4)) * 16;
     };
     {
         // exact division of a sample index below 4096 by gz: multiply and shift
-        if ((long long)k.slots * k.NZ >= 4096) return FBEV_ERR_TOO_LARGE;
+        if ((long long)k.slots_a * k.NZ >= 4096) return FBEV_ERR_TOO_LARGE;
         int l = 0;
         while ((1 << l) < k.gz) ++l;
         k.gz_shift = 12 + l;
@@ -212,16 +231,18 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
         hipLaunchKernelGGL(kernel, grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt);
         return true;
     };
-    bool ok;
-    if (stream) {
-        constexpr bool S = VEC > 1;      // no streaming instantiations off the vector paths
-        ok = pl.cpl == 1 ? launch(fbev_forward_kernel<T, VEC, 1, S>)
-                         : (pl.cpl == 2 ? launch(fbev_forward_kernel<T, VEC, 2, S>) : launch(fbev_forward_kernel<T, VEC, 4, S>));
-    } else {
-        ok = pl.cpl == 1 ? launch(fbev_forward_kernel<T, VEC, 1, false>)
-                         : (pl.cpl == 2 ? launch(fbev_forward_kernel<T, VEC, 2, false>)
-                                        : launch(fbev_forward_kernel<T, VEC, 4, false>));
-    }
+    // (batches of several groups and streamed output exist on the vector paths only; the plan asks for
+    // neither elsewhere)
+    constexpr bool V = VEC > 1;
+    const bool batched = V && pl.k.batch_groups > 1;
+    if (!V && pl.k.batch_groups > 1) return FBEV_ERR_LAUNCH;
+    auto pick = [&](auto cpl_tag) {
+        constexpr int CPL = decltype(cpl_tag)::value;
+        if (stream) return batched ? launch(fbev_forward_kernel<T, VEC, CPL, V, V>) : launch(fbev_forward_kernel<T, VEC, CPL, V, false>);
+        return batched ? launch(fbev_forward_kernel<T, VEC, CPL, false, V>) : launch(fbev_forward_kernel<T, VEC, CPL, false, false>);
+    };
+    const bool ok = pl.cpl == 1 ? pick(std::integral_constant<int, 1>{})
+                                : (pl.cpl == 2 ? pick(std::integral_constant<int, 2>{}) : pick(std::integral_constant<int, 4>{}));
     if (!ok) return FBEV_ERR_LAUNCH;
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
@@ -298,15 +319,62 @@ int launch_cells(const Plan &pl, const float *go, const void *depth, const void 
     const T *f = static_cast<const T *>(feats);
     const size_t lds = FILL ? pl.lds_fill : pl.lds_bwd;
     prof::Scope timer(FILL ? prof::kBackwardCells : prof::kBackwardScatter, st);
-    switch (pl.cpl) {
-        case 1: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 1, FILL>, lds)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 1, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride); break;
-        case 2: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 2, FILL>, lds)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 2, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride); break;
-        default: if (!lds_opt_in(fbev_backward_cells_kernel<T, VEC, 4, FILL>, lds)) return FBEV_ERR_LAUNCH;
-                hipLaunchKernelGGL((fbev_backward_cells_kernel<T, VEC, 4, FILL>), grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride); break;
-    }
+    constexpr bool V = VEC > 1;
+    const bool batched = V && pl.k.batch_groups > 1;
+    if (!V && pl.k.batch_groups > 1) return FBEV_ERR_LAUNCH;
+    auto launch = [&](auto kernel) {
+        if (!lds_opt_in(kernel, lds)) return false;
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride);
+        return true;
+    };
+    auto pick = [&](auto cpl_tag) {
+        constexpr int CPL = decltype(cpl_tag)::value;
+        return batched ? launch(fbev_backward_cells_kernel<T, VEC, CPL, FILL, V>) : launch(fbev_backward_cells_kernel<T, VEC, CPL, FILL, false>);
+    };
+    const bool ok = pl.cpl == 1 ? pick(std::integral_constant<int, 1>{})
+                                : (pl.cpl == 2 ? pick(std::integral_constant<int, 2>{}) : pick(std::integral_constant<int, 4>{}));
+    if (!ok) return FBEV_ERR_LAUNCH;
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
+}
+
+// Whether the batched cell pass pays for this instantiation: it holds a few more registers than the
+// plain one, and where those cost a wavefront per SIMD (512 registers per lane, allocated in eights)
+// the plain kernel is the faster one (training size, fp16: 101 against 91 registers, 4 against 5
+// wavefronts per SIMD, 397 against 385 us).  Asked of the runtime once per instantiation.
+int kernel_registers(const void *kernel) {
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, kernel) != hipSuccess) return 0;
+    return attr.numRegs;
+}
+
+template <typename T, int VEC, int FILL>
+bool cells_batch_pays_for(int cpl) {
+    static std::atomic<int> cache[3] = {{-1}, {-1}, {-1}};
+    const int idx = cpl == 1 ? 0 : (cpl == 2 ? 1 : 2);
+    int got = cache[idx].load(std::memory_order_relaxed);
+    if (got < 0) {
+        auto waves = [](int regs) { return regs > 0 ? 512 / ((regs + 7) / 8 * 8) : 0; };
+        auto both = [&](auto cpl_tag) {
+            constexpr int CPL = decltype(cpl_tag)::value;
+            const int with = kernel_registers(reinterpret_cast<const void *>(fbev_backward_cells_kernel<T, VEC, CPL, FILL, true>));
+            const int without = kernel_registers(reinterpret_cast<const void *>(fbev_backward_cells_kernel<T, VEC, CPL, FILL, false>));
+            return (with > 0 && without > 0 && waves(with) >= waves(without)) ? 1 : 0;
+        };
+        got = cpl == 1 ? both(std::integral_constant<int, 1>{})
+                       : (cpl == 2 ? both(std::integral_constant<int, 2>{}) : both(std::integral_constant<int, 4>{}));
+        cache[idx].store(got, std::memory_order_relaxed);
+    }
+    return got != 0;
+}
+
+template <int FILL>
+bool cells_batch_pays(const fbev_problem *p, const Plan &pl) {
+    if (pl.vec == 1) return false;
+    switch (p->in_dtype) {
+        case FBEV_F32: return cells_batch_pays_for<float, 4, FILL>(pl.cpl);
+        case FBEV_F16: return cells_batch_pays_for<__half, 8, FILL>(pl.cpl);
+        default: return cells_batch_pays_for<bf16_raw, 8, FILL>(pl.cpl);
+    }
 }
 
 template <int FILL>
@@ -442,8 +510,19 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     size_t cap64 = (workspace_bytes - index_bytes) / sizeof(Pair);
     const int cap = cap64 > 0x7fffffffull ? 0x7fffffff : (int)cap64;
     Plan pl;
-    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl, kCellPassWaves);
+    const bool allow_vec = (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0;
+    rc = make_plan(p, allow_vec, &pl, kCellPassWaves);
     if (rc != FBEV_OK) return rc;
+    {
+        // the cell pass in batches of several groups only where that does not cost occupancy
+        const long long tx = texel_count(p);
+        const bool fixed_layout = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (tx * kFixedReplicas) >= kFixedMinSegment;
+        const bool runs = sample_count(p) / (fixed_layout ? tx * kFixedReplicas : counter_count(p)) >= kClaimRunsFrom;
+        if (pl.k.batch_groups > 1 && !(runs ? cells_batch_pays<2>(p, pl) : cells_batch_pays<1>(p, pl))) {
+            rc = make_plan(p, allow_vec, &pl, kCellPassWaves, 3, kMaxSlotLdsBytes, 1);
+            if (rc != FBEV_OK) return rc;
+        }
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     char *base = static_cast<char *>(workspace);
     int *cursor = persistent ? reinterpret_cast<int *>(base + lay.sets) : static_cast<int *>(workspace);
@@ -649,6 +728,9 @@ int fbev_backward(const fbev_problem *p, const float *grad_out, const void *dept
     if (!d_depth && !d_feats) return FBEV_OK;
     Plan pl;
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl, kCellPassWaves);
+    if (rc == FBEV_OK && pl.k.batch_groups > 1 && !cells_batch_pays<0>(p, pl))
+        rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0, &pl, kCellPassWaves, 3,
+                       kMaxSlotLdsBytes, 1);
     if (rc != FBEV_OK) return rc;
     if (!accumulate) {
         rc = launch_zero(nullptr, 0, d_depth, texel_count(p) * p->depth_bins, d_feats, texel_count(p) * p->channels,

@@ -6,9 +6,12 @@
 namespace {
 
 // LDS of one block of the cell-centric kernels (float4 units):
-//   [matrices: N*12 floats][column table: slots*N ints][height table: gz floats]
-//   per wavefront: [16 ints of list lengths][16 float4 of cell centres][slots*N column records]
-//   [slots*N ints: columns in view][slots*NZ ints of candidates][slots * list_cap entries]
+//   [matrices: N*12 floats][column table: batch*N ints][height table: gz floats]
+//   per wavefront: [batch ints: entries per cell][batch ints: where a cell's entries start][8 ints: candidates
+//   before each group][batch float4 of cell centres][batch*N column records][batch*N ints: columns in view]
+//   [batch*NZ ints of candidates][pool of pool_cap entries]
+// where batch = KParams::slots_a cells go through the sample phase together and their kept samples
+// share one pool of entries, each cell's entries in one contiguous stretch.
 // Counters that several lanes of a wavefront update in turn live in LDS and are read as
 // volatile.  The pointer carries the LDS address space: a volatile access through a generic
 // pointer becomes a system-coherent flat load that first waits for every outstanding global
@@ -17,36 +20,45 @@ using lds_counter = volatile __attribute__((address_space(3))) int;
 
 struct WaveLds {
     const float *Pm;
-    const int *dec;       // column index within the wavefront's round -> slot << 28 | camera << 16
+    const int *dec;       // column index within the wavefront's batch -> cell << 28 | camera << 16
     const float *zt;      // height bin -> z of the bin's centre
-    lds_counter *cnt;     // entries per slot
-    float4 *cell;         // per slot: x, y, valid flag, ix | iy << 16
+    lds_counter *cnt;     // entries per cell of the batch
+    lds_counter *start;   // first entry of each cell in the pool
+    lds_counter *gcand;   // candidates that come before each group of the batch (groups + 1 values)
+    float4 *cell;         // per cell: x, y, valid flag, ix | iy << 16
     float4 *col;          // per column: the (x, y) part of U, V, D, and its dec word
     int *alive;           // columns with a height bin that may be in view
     unsigned *cand;       // samples that survive the cheap test: column << 16 | height bin
-    float4 *lst;
+    float4 *lst;          // the pool
 };
 
 __device__ __forceinline__ int lds_p_f4(const KParams &k) { return (k.N * 12 + 3) / 4; }
-__device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots * k.N + 3) / 4; }
-__device__ __forceinline__ int lds_cand_f4(const KParams &k) { return (k.slots * k.NZ + 3) / 4; }
+__device__ __forceinline__ int lds_dec_f4(const KParams &k) { return (k.slots_a * k.N + 3) / 4; }
+__device__ __forceinline__ int lds_cand_f4(const KParams &k) { return (k.slots_a * k.NZ + 3) / 4; }
 __device__ __forceinline__ int lds_z_f4(const KParams &k) { return (k.gz + 3) / 4; }
+// the three small tables and the cell records (LDS is granted in large granules: a few hundred bytes
+// per wavefront decide whether a tenth block fits a CU at the training size)
+__device__ __forceinline__ int lds_tables_f4(const KParams &k) { return (2 * k.slots_a + 8 + 3) / 4; }
+__device__ __forceinline__ int lds_head_f4(const KParams &k) { return lds_tables_f4(k) + k.slots_a; }
 
 // The wavefront's view of the block's LDS (pointers only).
 __device__ __forceinline__ WaveLds wave_lds_view(const KParams &k, float4 *smem, int entry_f4) {
     WaveLds L;
-    const int dec_f4 = lds_dec_f4(k), cand_f4 = lds_cand_f4(k), cols = k.slots * k.N;
-    const int per_wave_f4 = 4 + 16 + cols + dec_f4 + cand_f4 + k.slots * k.list_cap * entry_f4;
+    const int dec_f4 = lds_dec_f4(k), cand_f4 = lds_cand_f4(k), cols = k.slots_a * k.N;
+    const int head_f4 = lds_head_f4(k);
+    const int per_wave_f4 = head_f4 + cols + dec_f4 + cand_f4 + k.pool_cap * entry_f4;
     float4 *wbase = smem + lds_p_f4(k) + dec_f4 + lds_z_f4(k) + (threadIdx.x >> 6) * per_wave_f4;
     L.Pm = reinterpret_cast<float *>(smem);
     L.dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
     L.zt = reinterpret_cast<float *>(smem + lds_p_f4(k) + dec_f4);
     L.cnt = (lds_counter *)reinterpret_cast<int *>(wbase);
-    L.cell = wbase + 4;
-    L.col = wbase + 20;
-    L.alive = reinterpret_cast<int *>(wbase + 20 + cols);
-    L.cand = reinterpret_cast<unsigned *>(wbase + 20 + cols + dec_f4);
-    L.lst = wbase + 20 + cols + dec_f4 + cand_f4;
+    L.start = L.cnt + k.slots_a;
+    L.gcand = L.cnt + 2 * k.slots_a;
+    L.cell = wbase + lds_tables_f4(k);
+    L.col = wbase + head_f4;
+    L.alive = reinterpret_cast<int *>(wbase + head_f4 + cols);
+    L.cand = reinterpret_cast<unsigned *>(wbase + head_f4 + cols + dec_f4);
+    L.lst = wbase + head_f4 + cols + dec_f4 + cand_f4;
     return L;
 }
 
@@ -58,7 +70,7 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
     float *Pm = reinterpret_cast<float *>(smem);
     int *dec = reinterpret_cast<int *>(smem + lds_p_f4(k));
     float *zt = reinterpret_cast<float *>(smem + lds_p_f4(k) + lds_dec_f4(k));
-    const int cols = k.slots * k.N;
+    const int cols = k.slots_a * k.N;
     for (int i = threadIdx.x; i < k.N * 12; i += blockDim.x)
         Pm[i] = proj[(size_t)(b * k.N + i / 12) * k.proj_stride + (i % 12)];
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
@@ -88,7 +100,7 @@ enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeF
 // the exact test it would otherwise take (and fail).
 constexpr float kEarlySlack = 1.0e-3f;
 
-// Phase A of one round of a wavefront: the samples of its `slots` cells, in three stages.
+// The sample phase of one batch of a wavefront: the samples of its `slots_a` cells, in three stages.
 //   stage 0  lanes = (cell, camera) columns: the (x, y) part of the three dot products, shared by
 //            the column's height bins, and a test of the column's two end bins.  U, V and D are
 //            monotone in the height bin (every rounded operation is), so a column whose end bins
@@ -100,17 +112,22 @@ constexpr float kEarlySlack = 1.0e-3f;
 //            in order, into the candidate list.
 //   stage 2  lanes = candidates, densely packed: the canonical arithmetic (divisions, floor,
 //            bilinear weights), the depth model, the weight threshold; what is kept goes, still
-//            in (camera, height) order, into its slot's entry list.
-// kModeCount writes no entries; it only counts the kept samples per (first-corner texel, replica).
-template <int ENTRY_F4, typename T, int MODE>
-__device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, const T *__restrict__ depth, int b, int q0,
-                                        int lane, const int *__restrict__ chunk_prefix = nullptr,
-                                        int *__restrict__ cursor = nullptr, int pair_cap = 0) {
-    constexpr bool FILLING = MODE == kModeFill || MODE == kModeFillRuns;   // the latter claims per run
-    constexpr bool BACKWARD = MODE == kModeScatter || FILLING;
-    const int n_cols = k.slots * k.N;
-    if (lane < 16) L.cnt[lane] = 0;
-    if (lane < k.slots) {
+//            in (cell, camera, height) order, into the pool of entries.
+// A batch is `batch_groups` groups of `slots` cells: phase B works on one group at a time (its lane
+// groups cover `slots` cells), while stages 0 to 2 run over the whole batch, so that their passes
+// of 64 lanes are filled by more than one group's samples (a group of two cells has about thirty
+// candidates: stage 2, a third of the forward's instructions, ran at half its lanes).  The pool holds
+// slots * NZ entries, what one group can keep at most; when a batch has more candidates than that
+// (rare: about one sample in six is in view), its groups go through stage 2 one at a time.
+
+// Stages 0 and 1 of the batch that starts at cell q0.  Returns the number of candidates; the number
+// of candidates before each group is left in L.gcand.
+// BATCHED = false is the batch of one group, with the bookkeeping of several compiled away.
+template <bool BATCHED>
+__device__ __forceinline__ int phase_a_candidates(const KParams &k, const WaveLds &L, int q0, int lane) {
+    const int n_groups = BATCHED ? k.batch_groups : 1;
+    const int n_cols = k.slots_a * k.N;
+    if (lane < k.slots_a) {
         int ix = 0, iy = 0;
         const bool ok = cell_of(k, q0 + lane, ix, iy);
         L.cell[lane] = make_float4(voxel_coord(k.xmin, ix, k.vx), voxel_coord(k.ymin, iy, k.vy), ok ? 1.0f : 0.0f,
@@ -154,16 +171,19 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
 
     // ---- stage 1
     int n_cand = 0;
+    int before1 = 0, before2 = 0, before3 = 0;      // candidates of groups below 1, 2, 3 (at most four groups)
     const int total = n_alive * k.gz;
     for (int base = 0; base < total; base += kWave) {
         const int idx = base + lane;
         bool pass = false;
         unsigned key = 0;
+        int cell = 0;
         if (idx < total) {
             const int a = (int)(__umul24((unsigned)idx, (unsigned)k.gz_magic) >> k.gz_shift);
             const int iz = idx - a * k.gz;
             const int cc = L.alive[a];
             const float4 col = L.col[cc];
+            cell = (__float_as_int(col.w) >> 28) & 15;
             const float *P = L.Pm + ((__float_as_int(col.w) >> 16) & 0xfff) * 12;
             const float z = L.zt[iz];
             const float D = (col.z + P[10] * z) + P[11];
@@ -178,18 +198,46 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         const unsigned long long m = __ballot(pass);
         if (pass) L.cand[n_cand + __popcll(m & lanemask_lt(lane))] = key;
         n_cand += __popcll(m);
+        if (BATCHED) {
+            before1 += __popcll(__ballot(pass && cell < k.slots));
+            before2 += __popcll(__ballot(pass && cell < 2 * k.slots));
+            before3 += __popcll(__ballot(pass && cell < 3 * k.slots));
+        }
+    }
+    if (BATCHED && lane == 0) {
+        L.gcand[0] = 0;
+        L.gcand[1] = before1;
+        L.gcand[2] = before2;
+        L.gcand[3] = before3;
+        L.gcand[n_groups] = n_cand;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    return n_cand;
+}
 
-    // ---- stage 2
-    for (int base = 0; base < n_cand; base += kWave) {
+// Stage 2 over the candidates [c_lo, c_hi) of the batch (whole groups).  Entries are appended to the
+// pool from its start; on return L.cnt holds the entries of every cell (0 for the cells of other
+// groups) and L.start where they begin.
+// kModeCount writes no entries; it only counts the kept samples per (first-corner texel, replica).
+template <int ENTRY_F4, typename T, int MODE>
+__device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds &L, const T *__restrict__ depth, int b,
+                                                int lane, int c_lo, int c_hi,
+                                                const int *__restrict__ chunk_prefix = nullptr,
+                                                int *__restrict__ cursor = nullptr, int pair_cap = 0) {
+    constexpr bool FILLING = MODE == kModeFill || MODE == kModeFillRuns;   // the latter claims per run
+    constexpr bool BACKWARD = MODE == kModeScatter || FILLING;
+    if (lane < k.slots_a) L.cnt[lane] = 0;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    int n_pool = 0;       // entries in the pool so far
+    for (int base = c_lo; base < c_hi; base += kWave) {
         const int j = base + lane;
-        const bool active = j < n_cand;
+        const bool active = j < c_hi;
         const unsigned key = active ? L.cand[j] : 0u;
         const float4 col = active ? L.col[key >> 16] : make_float4(0.f, 0.f, 0.f, 0.f);
         const int d = __float_as_int(col.w);
-        const int slot = active ? (d >> 28) & 15 : 16 + (lane & 1);   // idle lanes: no real slot
+        const int slot = active ? (d >> 28) & 15 : 16 + (lane & 1);   // idle lanes: no real cell
         const int cam = (d >> 16) & 0xfff;
         float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w2 = w0;
         int4 tx = make_int4(0, 0, 0, 0);
@@ -265,10 +313,13 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
         const unsigned long long above = lane == 63 ? 0ull : (bm & ~lanemask_le(lane));
         const int hi = above ? __ffsll((long long)above) - 1 : kWave;
         const unsigned long long seg = (~0ull << lo) & (hi >= 64 ? ~0ull : ((1ull << hi) - 1ull));
-        const int prefix = __popcll(m & seg & lanemask_lt(lane));
         const int old = active ? L.cnt[slot] : 0;
-        if (keep) {
-            float4 *e = L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4;
+        // kept samples are appended to the pool in order: a cell's entries end up next to each other
+        // (`at` of a lane that keeps nothing is where the next kept sample after it goes)
+        const int at = n_pool + __popcll(m & lanemask_lt(lane));
+        n_pool += __popcll(m);
+        if (keep && ENTRY_F4 > 0) {
+            float4 *e = L.lst + (size_t)at * ENTRY_F4;
             e[0] = w0;
             if (ENTRY_F4 > 1)
                 e[1] = BACKWARD ? w2
@@ -289,7 +340,7 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                 pos = atomicAdd(cursor + i0, 1);
                 pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
             }
-            reinterpret_cast<int *>(L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4)[3] = pos;
+            reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
         }
         if (MODE == kModeFillRuns) {
             // the same, but the run's first lane claims for the whole run (same cell and texel: same
@@ -307,10 +358,15 @@ __device__ __forceinline__ void phase_a(const KParams &k, const WaveLds &L, cons
                 } else {
                     pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
                 }
-                reinterpret_cast<int *>(L.lst + (size_t)(slot * k.list_cap + old + prefix) * ENTRY_F4)[3] = pos;
+                reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
             }
         }
-        if (active && lane == lo) L.cnt[slot] = old + __popcll(m & seg);
+        if (active && lane == lo) {
+            // the first lane of a cell's stretch of lanes keeps the cell's books: its entries so far, and,
+            // when these are its first, where they start in the pool (a cell without entries has no start)
+            L.cnt[slot] = old + __popcll(m & seg);
+            if (old == 0) L.start[slot] = at;
+        }
     }
 }
 
