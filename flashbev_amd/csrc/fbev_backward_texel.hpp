@@ -67,15 +67,9 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     constexpr int n_waves = WAVES;
     const bool counted = chunk_prefix != nullptr;
     const bool persistent = ps.epoch != nullptr;
-    if (persistent) {
-        const int epoch = ps.epoch[0], set = epoch & 1;
-        seg_end = ps.sets + (size_t)set * ps.set_stride;
-        if (threadIdx.x == 0 && blockIdx.y == 0) {
-            // the counters of this texel in the set the next call claims in
-            *reinterpret_cast<int4 *>(ps.sets + (size_t)(set ^ 1) * ps.set_stride + (size_t)t * kFixedReplicas) = make_int4(0, 0, 0, 0);
-            if (blockIdx.x == 0) ps.epoch[1] = epoch + 1;
-        }
-    }
+    // (persistent: which set of counters this call claimed in; the lists' bounds are requested
+    // from both sets before the answer is needed)
+    const int epoch = persistent ? ps.epoch[0] : 0, set = epoch & 1;
     // List e of the texel: first corner (e & 3 with fixed segments, e when counted): bit 0 = one
     // texel to the left, bit 1 = one row up; replica e >> 2 with fixed segments.  A cell's samples
     // on neighbouring height bins sit in different lists of the same replica, at about the same
@@ -103,10 +97,21 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             // fixed segments of pair_cap pairs; seg_end holds how many were claimed
             const int i = q * kFixedReplicas + (e >> 2);
             my_lo = i * pair_cap;
-            const int claimed = seg_end[i];
+            int claimed;
+            if (persistent) {
+                const int in_first = ps.sets[i], in_second = ps.sets[ps.set_stride + i];
+                claimed = set ? in_second : in_first;
+            } else {
+                claimed = seg_end[i];
+            }
             spilled = claimed > pair_cap;
             my_len = max(min(claimed, pair_cap), 0);
         }
+    }
+    if (persistent && threadIdx.x == 0 && blockIdx.y == 0) {
+        // the counters of this texel in the set the next call claims in
+        *reinterpret_cast<int4 *>(ps.sets + (size_t)(set ^ 1) * ps.set_stride + (size_t)t * kFixedReplicas) = make_int4(0, 0, 0, 0);
+        if (blockIdx.x == 0) ps.epoch[1] = epoch + 1;
     }
     // the lists one after the other form one sequence of pairs; list e starts at my_pre of lane e
     int my_pre = my_len;
