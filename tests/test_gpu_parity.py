@@ -13,6 +13,7 @@ import numpy as np
 import pytest
 import torch
 
+from flashbev_amd import capi
 from flashbev_amd.workloads import WORKLOADS, make_inputs
 from oracle import c_oracle, dense_torch
 from tests import _util as U
@@ -87,6 +88,40 @@ def test_backward_single_gradient():
         assert df is None and U.violations(dd.cpu().numpy(), want_dd)[0] == 0
         dd, df = U.capi_backward(x, w, 0, mode=mode, want=(False, True))
         assert dd is None and U.violations(df.cpu().numpy(), want_df)[0] == 0
+
+
+def test_one_persistent_workspace_through_calls_of_different_kinds():
+    """A workspace prepared once serves calls that ask for one gradient or for both, that overwrite
+    or accumulate, under either parametric depth model: every call must leave the claim counters and
+    the workspace's own gradient buffers ready for the next, whatever that one asks for."""
+    w, x = _inputs("cfg2_surround", 0)
+    want = {dist: U.oracle_backward(x, w, dist) for dist in (0, 1)}
+    dev = x["image_feats"].device
+    st = torch.cuda.current_stream().cuda_stream
+    p0 = U.problem_for(x, w, 0)
+    nbytes = capi.backward_persistent_workspace_bytes(p0)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(0x5A)
+    capi.check(capi.backward_workspace_init(p0, ws.data_ptr(), nbytes, st), "fbev_backward_workspace_init")
+    # (depth model, depth gradient?, feature gradient?, accumulate onto ones?)
+    calls = [(0, True, True, False), (0, True, False, False), (1, False, True, False), (1, True, True, True),
+             (0, False, True, True), (1, True, False, False), (0, True, True, False)]
+    for dist, need_dd, need_df, accumulate in calls:
+        p = U.problem_for(x, w, dist)
+        fill = 1.0 if accumulate else float("nan")
+        dd = torch.full(x["depth_params"].shape, fill, dtype=torch.float32, device=dev) if need_dd else None
+        df = torch.full(x["image_feats"].shape, fill, dtype=torch.float32, device=dev) if need_df else None
+        capi.check(capi.backward_gather_persistent(
+            p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
+            x["projection_matrices"].data_ptr(), dd.data_ptr() if need_dd else None, df.data_ptr() if need_df else None,
+            ws.data_ptr(), nbytes, st, accumulate=accumulate), "fbev_backward_gather_persistent")
+        torch.cuda.synchronize()
+        for got, ref, what in ((dd, want[dist][0], "d_depth"), (df, want[dist][1], "d_feats")):
+            if got is None:
+                continue
+            got = got.double().cpu().numpy() - (1.0 if accumulate else 0.0)
+            # (a sum that was added to 1.0 carries half an ulp of 1.0 on top of the stated tolerance)
+            bad = np.abs(got - ref) > 1e-5 + 1e-4 * np.abs(ref) + (1e-7 if accumulate else 0.0)
+            assert not bad.any(), (dist, need_dd, need_df, accumulate, what, int(bad.sum()))
 
 
 @pytest.mark.parametrize("dist", [0, 1])
