@@ -13,6 +13,9 @@ parameters, tools/config/config.yaml:29).  The single JSON line printed on stdou
                         synchronisations; ms_per_step_graph is the same step captured into a HIP
                         graph and replayed K times (checked against the eager result first) --
                         on this machine the eager queue is already GPU-bound and no slower
+  sustain_ms            every timing is preceded by this many milliseconds of untimed steps of its own
+                        workload (then the W warm-up steps): from idle the GPU needs 10-30 ms of
+                        continuous work to reach the clocks it holds afterwards
   roofline              the dominant pass (the backward: cell pass + texel pass): its compulsory
                         bytes / the summed mean durations of its kernels, measured with HIP
                         events the library records around every one of its launches over a
@@ -117,6 +120,24 @@ class Runner:
             self.counts, False, self.workspace)
 
 
+# Untimed steps of the workload itself, run for this many milliseconds before the warm-up steps of every
+# timing below.  From idle the GPU needs 10-30 ms of continuous work to reach the clocks it then holds
+# (measured per 2 ms of steps from idle: 48.1, 47.2, 46.7, 46.0, then 45.5 us per step for good); without this
+# a short run times the ramp.  --sustain-ms 0 switches it off.
+SUSTAIN_MS = 50.0
+
+
+def sustain(step, ms=None):
+    ms = SUSTAIN_MS if ms is None else ms
+    if ms <= 0:
+        return
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(8):
+            step()
+        torch.cuda.synchronize()
+
+
 def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
     """Wall-clock over exactly `steps` eagerly queued steps (nothing but the operator's launches
     between the two synchronisations), then the same steps again with events around each pass
@@ -126,6 +147,7 @@ def time_steps(r: Runner, steps: int, warmup: int, with_backward: bool):
         if with_backward:
             r.backward()
 
+    sustain(step)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -160,6 +182,7 @@ def time_cached_forward(r: Runner, steps: int, warmup: int):
     torch.cuda.synchronize()
     if not torch.equal(r.out, want):
         raise RuntimeError("forward on cached geometry differs from the forward")
+    sustain(lambda: r.forward(cache))
     for _ in range(warmup):
         r.forward(cache)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
@@ -203,6 +226,7 @@ def time_graph_steps(r: Runner, steps: int, warmup: int):
                 if not torch.allclose(got, ref, rtol=1e-4, atol=1e-5):
                     raise RuntimeError(f"graph replay {i}: {what} differs from the eager result")
     torch.cuda.synchronize()
+    sustain(graph.replay)
     t0 = time.perf_counter()
     for _ in range(steps):
         graph.replay()
@@ -231,6 +255,7 @@ def time_operator_steps(r: Runner, steps: int, warmup: int):
             else:
                 feats.grad = depth.grad = None
                 flash_bevpool(image_feats=feats, depth_params=depth, **kw).backward(x["grad_out"])
+        sustain(step)
         for _ in range(max(warmup, 10)):
             step()
         torch.cuda.synchronize()
@@ -374,12 +399,15 @@ def run_table(steps: int, warmup: int, out_dir: str):
 
 
 def main():
+    global SUSTAIN_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2_surround", choices=sorted(WORKLOADS))
     ap.add_argument("--depth", default="laplace", choices=sorted(DIST_OF))
+    ap.add_argument("--sustain-ms", type=float, default=SUSTAIN_MS,
+                    help="untimed steps run for this long before each timing's warm-up, to reach sustained clocks (0 = off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--table", action="store_true")
     ap.add_argument("--table-dir", default="bench_out", help="directory (under the repository) for the --table files")
@@ -394,6 +422,7 @@ def main():
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="only run a device-to-device copy of this many MiB (counter calibration)")
     args = ap.parse_args()
+    SUSTAIN_MS = args.sustain_ms
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; batch elements are independent, so more GPUs "
               "would each take a slice of the batch with no exchange. Run with --gpus 1.", file=sys.stderr)
@@ -418,6 +447,7 @@ def main():
         # for profilers: nothing but warm-up and timed steps of the one workload (every launch of the run
         # belongs to it), optionally with the forward on cached geometry in place of the forward
         cache = r.geometry_cache() if args.only_steps == "cached" else None
+        sustain(lambda: (r.forward(cache), r.backward()))
         for _ in range(args.warmup):
             r.forward(cache); r.backward()
         torch.cuda.synchronize()
@@ -457,6 +487,7 @@ def main():
         "metric": "BEV-pool fwd+bwd latency (ms) & effective HBM GB/s, 6 cams 128x128xZ=8, 1 GPU",
         "value": ms, "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "sustain_ms": SUSTAIN_MS,
         "dtype": "f32" if w.dtype == torch.float32 else str(w.dtype).replace("torch.", ""),
         "data": "synthetic",
         "config": {"workload": w.name, "depth_model": args.depth, "batch": w.batch, "cams": w.num_cams,
