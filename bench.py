@@ -408,6 +408,8 @@ def main():
     ap.add_argument("--depth", default="laplace", choices=sorted(DIST_OF))
     ap.add_argument("--sustain-ms", type=float, default=SUSTAIN_MS,
                     help="untimed steps run for this long before each timing's warm-up, to reach sustained clocks (0 = off)")
+    ap.add_argument("--ramp", action="store_true",
+                    help="print how the step time of --workload settles from idle (slices of steps after 0.5 s without GPU work)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--table", action="store_true")
     ap.add_argument("--table-dir", default="bench_out", help="directory (under the repository) for the --table files")
@@ -443,6 +445,26 @@ def main():
         print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n}))
         return
     r = Runner(w, args.depth, backward_mode=args.backward_mode)
+    if args.ramp:
+        # how the step time settles from idle: the mean over consecutive slices of steps after half a
+        # second without GPU work (what sustain_ms is sized by)
+        for _ in range(3):
+            r.forward(); r.backward()
+        torch.cuda.synchronize()
+        time.sleep(0.5)
+        per_slice = max(1, int(round(2.0 / 0.045))) if w.name in ("cfg1_tiny", "cfg2_surround") else 10
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(41)]
+        ev[0].record()
+        for i in range(40):
+            for _ in range(per_slice):
+                r.forward(); r.backward()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(40)]
+        print(json.dumps({"workload": w.name, "depth_model": args.depth, "steps_per_slice": per_slice,
+                          "us_per_step_by_slice": [round(v / per_slice * 1e3, 1) for v in ms],
+                          "ms_since_start_at_slice_end": [round(sum(ms[:i + 1]), 1) for i in range(40)]}), flush=True)
+        return
     if args.only_steps:
         # for profilers: nothing but warm-up and timed steps of the one workload (every launch of the run
         # belongs to it), optionally with the forward on cached geometry in place of the forward
