@@ -100,7 +100,7 @@ def _persistent_workspace(ext, depth_params, image_feats, projection_matrices, f
     return key, ws
 
 
-# id(tensor) -> (weak reference, version, values).  Keyed by identity: a mapping keyed by the
+# id(tensor) -> (weak reference, version, values, notes about the values).  Keyed by identity: a mapping keyed by the
 # tensors themselves would compare them with ``==`` on lookup, which is elementwise.
 _host_cache: dict = {}
 
@@ -114,23 +114,22 @@ def _device_values(x):
         return hit[2]
     vals = x.detach().reshape(-1).tolist()
     ref = weakref.ref(x, lambda _r, key=key: _host_cache.pop(key, None))
-    _host_cache[key] = (ref, x._version, vals)
+    _host_cache[key] = (ref, x._version, vals, {})
     return vals
 
 
-def _host_values(x, n: int, name: str):
-    """Values of a small size/range argument as Python numbers.  Sequences and CPU tensors cost
-    nothing; a device tensor costs one synchronous copy the first time it is seen."""
+def _host_values(x, n: int, name: str, conv=float):
+    """A small size/range argument as a tuple of Python numbers.  Sequences cost nothing; a tensor is
+    read the first time it is seen (a device tensor with one synchronous copy)."""
     if isinstance(x, torch.Tensor):
         if x.numel() != n:
             raise ValueError(f"{name} must have {n} elements, got shape {tuple(x.shape)}")
-        if x.device.type == "cpu":
-            return x.reshape(-1).tolist()
-        return _device_values(x)
-    vals = list(x)
-    if len(vals) != n:
-        raise ValueError(f"{name} must have {n} elements, got {len(vals)}")
-    return vals
+        vals = x.reshape(-1).tolist() if x.device.type == "cpu" else _device_values(x)
+    else:
+        vals = x if isinstance(x, (list, tuple)) else list(x)
+        if len(vals) != n:
+            raise ValueError(f"{name} must have {n} elements, got {len(vals)}")
+    return tuple(map(conv, vals))
 
 
 def _check_feature_size(feature_size, cameras: int, H: int, W: int):
@@ -140,19 +139,28 @@ def _check_feature_size(feature_size, cameras: int, H: int, W: int):
     sampling the padding.  ``None`` is accepted (the shape is used)."""
     if feature_size is None:
         return
+    notes = None
     if isinstance(feature_size, torch.Tensor):
         if feature_size.numel() != 2 * cameras:
             raise ValueError(f"feature_size must have shape [B, N, 2] = {2 * cameras} elements, got "
                              f"{tuple(feature_size.shape)}")
-        vals = (feature_size.reshape(-1).tolist() if feature_size.device.type == "cpu"
-                else _device_values(feature_size))
+        if feature_size.device.type == "cpu":
+            vals = feature_size.reshape(-1).tolist()
+        else:
+            # the values of a device tensor object and version are read once, and checked once per (H, W)
+            vals = _device_values(feature_size)
+            notes = _host_cache[id(feature_size)][3]
+            if notes.get("feature_size_ok") == (H, W):
+                return
     else:
         vals = [int(v) for row in feature_size for v in (row if hasattr(row, "__iter__") else [row])]
         if len(vals) != 2 * cameras:
             raise ValueError(f"feature_size must hold (H, W) for each of {cameras} cameras")
-    if any(int(vals[i]) != (H, W)[i & 1] for i in range(len(vals))):
+    if vals[0::2] != [H] * cameras or vals[1::2] != [W] * cameras:
         raise RuntimeError(f"feature_size must equal the feature maps' shape (H, W) = ({H}, {W}) for every "
                          f"camera; per-camera valid sizes inside a padded tensor are not supported")
+    if notes is not None:
+        notes["feature_size_ok"] = (H, W)
 
 
 def voxel_geometry(roi_range: Sequence[float], grid_size: Sequence[int]):
@@ -211,9 +219,9 @@ class FlashBEVPool(torch.autograd.Function):
         d_min, d_step = (1.0, 1.0) if depth_range is None else (float(depth_range[0]), float(depth_range[1]))
 
         B, N, H, W, C = image_feats.shape
-        grid = tuple(int(v) for v in _host_values(grid_size, 3, "grid_size"))
-        image = tuple(int(v) for v in _host_values(image_size, 2, "image_size"))
-        roi = tuple(float(v) for v in _host_values(roi_range, 6, "roi_range"))
+        grid = _host_values(grid_size, 3, "grid_size", int)
+        image = _host_values(image_size, 2, "image_size", int)
+        roi = _host_values(roi_range, 6, "roi_range", float)
         image_t, grid_t, roi_t, vmin, vsize = _host_arguments(grid, image, roi)
 
         # feature_size repeats the feature tensor's (H, W) per camera: checked (a device tensor is
@@ -234,16 +242,17 @@ class FlashBEVPool(torch.autograd.Function):
             bool(use_warp_kernel), bool(use_vectorized_load), float(epsilon),
             float(depth_weight_threshold), d_min, d_step, red, counts, geometry_cache)
 
-        ctx.save_for_backward(depth_params, image_feats, projection_matrices)
-        ctx.counts = counts
-        ctx.pair_capacity = _pair_capacity(B, N, grid)
-        ctx.host = (fs_host, image_t, roi_t, grid_t)
-        ctx.total_threads = out.numel()
-        ctx.depth_distribution = depth_distribution
-        ctx.epsilon = float(epsilon)
-        ctx.depth_weight_threshold = float(depth_weight_threshold)
-        ctx.depth_range = (d_min, d_step)
-        ctx.reduction = red
+        if wants_grad:
+            ctx.save_for_backward(depth_params, image_feats, projection_matrices)
+            ctx.counts = counts
+            ctx.pair_capacity = _pair_capacity(B, N, grid)
+            ctx.host = (fs_host, image_t, roi_t, grid_t)
+            ctx.total_threads = out.numel()
+            ctx.depth_distribution = depth_distribution
+            ctx.epsilon = float(epsilon)
+            ctx.depth_weight_threshold = float(depth_weight_threshold)
+            ctx.depth_range = (d_min, d_step)
+            ctx.reduction = red
         return out
 
     @staticmethod
@@ -292,11 +301,23 @@ def flash_bevpool(image_feats, depth_params, projection_matrices, feature_size, 
     (x,y,z).  Returns [B, Y, X, C] float32.  ``geometry_cache`` (from ``build_geometry_cache`` for the same
     matrices, sizes, grid and epsilon) lets the forward skip the projection; the result is the same bit for bit.
     """
-    return FlashBEVPool.apply(depth_params, image_feats, projection_matrices, feature_size,
-                              image_size, roi_range, grid_size, depth_distribution,
-                              use_shared_memory, optimize_z_precompute, use_warp_kernel,
-                              use_vectorized_load, epsilon, depth_weight_threshold, depth_range,
-                              reduction, geometry_cache)
+    args = (depth_params, image_feats, projection_matrices, feature_size, image_size, roi_range, grid_size,
+            depth_distribution, use_shared_memory, optimize_z_precompute, use_warp_kernel, use_vectorized_load,
+            epsilon, depth_weight_threshold, depth_range, reduction, geometry_cache)
+    if not (torch.is_grad_enabled() and (_wants_grad(depth_params) or _wants_grad(image_feats))):
+        # nothing to differentiate (inference): the same forward without the autograd function's bookkeeping,
+        # which costs more host time than a small forward takes on the GPU
+        return FlashBEVPool.forward(_NoGrad, *args)
+    return FlashBEVPool.apply(*args)
+
+
+def _wants_grad(x) -> bool:
+    return isinstance(x, torch.Tensor) and x.requires_grad
+
+
+class _NoGrad:
+    """Stands in for the autograd context when nothing is differentiated (the forward then leaves it alone)."""
+    needs_input_grad = (False,) * 17
 
 
 def build_geometry_cache(projection_matrices, feature_size, image_size, roi_range, grid_size, epsilon=1e-6):
@@ -312,9 +333,9 @@ def build_geometry_cache(projection_matrices, feature_size, image_size, roi_rang
     else:
         fs = [int(v) for row in feature_size for v in (row if hasattr(row, "__iter__") else [row])]
     H, W = int(fs[0]), int(fs[1])
-    grid = tuple(int(v) for v in _host_values(grid_size, 3, "grid_size"))
-    image = tuple(int(v) for v in _host_values(image_size, 2, "image_size"))
-    roi = tuple(float(v) for v in _host_values(roi_range, 6, "roi_range"))
+    grid = _host_values(grid_size, 3, "grid_size", int)
+    image = _host_values(image_size, 2, "image_size", int)
+    roi = _host_values(roi_range, 6, "roi_range", float)
     vmin, vsize = voxel_geometry(roi, grid)
     return ext.build_geometry_cache(projection_matrices.contiguous().float(), H, W, image[0], image[1], list(grid),
                                     vmin, vsize, float(epsilon))

@@ -248,6 +248,26 @@ def test_wrapper_puts_feats_first_and_skips_unneeded_grads(fake_ext):
     assert f.grad is not None
 
 
+def test_forward_without_gradients_skips_the_autograd_function(fake_ext, monkeypatch):
+    """Inference calls (no input requires a gradient, or gradients are switched off) run the same forward
+    without the autograd function around it: no sample counts are asked for and nothing is saved."""
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    base = (x["depth_params"], x["projection_matrices"], x["feature_size"], x["image_size"], x["roi_range"],
+            x["grid_size"])
+    applied = []
+    real_apply = FlashBEVPool.apply
+    monkeypatch.setattr(FlashBEVPool, "apply", lambda *a: applied.append(1) or real_apply(*a))
+    out = flash_bevpool(x["image_feats"], *base)
+    assert not applied and not out.requires_grad and fake_ext.fwd[-2] is None        # no count buffer
+    f = x["image_feats"].clone().requires_grad_(True)
+    with torch.no_grad():
+        out = flash_bevpool(f, *base)
+    assert not applied and not out.requires_grad
+    out = flash_bevpool(f, *base)
+    assert applied and out.requires_grad and fake_ext.fwd[-2] is not None
+
+
 def test_half_inputs_are_not_upcast_and_mixed_dtypes_are(fake_ext):
     w = WORKLOADS["cfg1_tiny"]
     x = make_inputs(w, "parametric")
