@@ -3,7 +3,9 @@ looking up, down and backwards), random intrinsics, off-centre and anisotropic g
 poses exercise what the benchmark rig does not: samples near the camera plane, projections that
 wrap around the image, tiles that straddle the field of view -- the cases the kernels' early
 rejection and the column backward's culling must get right.  Everything is compared with the C
-oracle: masks and indices bit for bit, outputs and gradients within 1e-5 + 1e-4 |ref|."""
+oracle: masks and indices bit for bit, outputs and gradients within 1e-5 + 1e-4 |ref|, in fp32, fp16
+and bf16 inputs by turns; the forward on cached geometry must repeat the forward's bits, and every
+backward algorithm and workspace kind must agree with the oracle."""
 import dataclasses
 import math
 
@@ -55,6 +57,11 @@ def test_random_rig(seed):
     P = np.stack([[random_pose(rng) for _ in range(n_cams)] for _ in range(batch)]).astype(np.float32)
     x["projection_matrices"] = torch.from_numpy(P).cuda().contiguous()
     thr = float(rng.choice([0.0, 1e-6, 1e-3]))
+    # a third of the cases in each input type (half-precision inputs are widened exactly, so the oracle
+    # runs on the same values and the tolerance does not change)
+    dtype = (torch.float32, torch.float16, torch.bfloat16)[seed % 3]
+    for name in ("image_feats", "depth_params"):
+        x[name] = x[name].to(dtype).contiguous()
 
     mask, idx, frac = U.capi_geometry(x["projection_matrices"], w)
     ref = c_oracle.geometry(P, w.feat_hw, w.image_hw, w.roi_range, w.grid_size)
@@ -67,8 +74,13 @@ def test_random_rig(seed):
     assert np.array_equal(cnt.cpu().numpy(), want_cnt), "per-cell sample counts differ"
     bad, maxabs, ratio = U.violations(out.cpu().numpy(), want)
     assert bad == 0, (bad, maxabs, ratio)
+    # the forward on cached geometry: the same bits
+    cache = U.capi_geometry_cache(x, w, dist)
+    got, got_cnt = U.capi_forward_cached(x, w, dist, cache, thr, with_count=True)
+    assert torch.equal(got, out) and torch.equal(got_cnt, cnt)
     want_dd, want_df = U.oracle_backward(x, w, dist, thr)
-    for mode in ("scatter", "gather", "gather_counted", "columns", "columns_acc", "gather_overwrite"):
+    for mode in ("scatter", "gather", "gather_counted", "columns", "columns_acc", "gather_overwrite",
+                 "persistent_overwrite"):
         dd, df = U.capi_backward(x, w, dist, thr, mode=mode)
         for got, r, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
             bad, maxabs, ratio = U.violations(got.cpu().numpy(), r)
