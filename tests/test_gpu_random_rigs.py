@@ -85,3 +85,48 @@ def test_random_rig(seed):
         for got, r, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
             bad, maxabs, ratio = U.violations(got.cpu().numpy(), r)
             assert bad == 0, f"seed {seed} {mode} {what}: {bad} outside tolerance (max {maxabs:.3e}, ratio {ratio:.2f})"
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes(seed):
+    """Wider shapes than the rigs above: up to 8 cameras, batches of 3, feature maps from 1x1 to 39x99, 1 to
+    512 channels (on and off the 128-bit path), grids up to 149x149x24, 2 to 129 depth bins, the benchmark
+    rig or arbitrary poses, fp32 / fp16 / bf16 inputs.  Counts exactly, outputs within 1e-5 + 1e-4 |ref|,
+    the forward on cached geometry bit for bit; gradients within 3e-5 + 3e-4 |ref| (a texel of a one-row
+    feature map can collect every sample of a camera: tens of thousands of fp32 terms in an order the
+    claims do not fix, against the oracle's float64 sums)."""
+    rng = np.random.default_rng(5000 + seed)
+    n_cams, batch = int(rng.integers(1, 9)), int(rng.integers(1, 4))
+    gx, gy, gz = int(rng.integers(8, 150)), int(rng.integers(8, 150)), int(rng.integers(1, 25))
+    cx, cy = rng.uniform(-10, 10, size=2)
+    roi = (cx - rng.uniform(10, 60), cx + rng.uniform(10, 60), cy - rng.uniform(10, 60), cy + rng.uniform(10, 60),
+           rng.uniform(-6, -1), rng.uniform(0.5, 5))
+    channels = int(rng.choice([1, 3, 4, 8, 20, 33, 64, 80, 128, 200, 256, 384, 512]))
+    dist = int(rng.integers(0, 3))
+    w = dataclasses.replace(WORKLOADS["cfg1_tiny"], batch=batch, yaws=tuple([0.0] * n_cams), channels=channels,
+                            feat_hw=(int(rng.integers(1, 40)), int(rng.integers(1, 100))), roi_range=roi,
+                            grid_size=(gx, gy, gz), depth_bins=int(rng.integers(2, 130)),
+                            depth_range=(float(rng.uniform(0.5, 3)), float(rng.uniform(0.25, 2.5))))
+    x = make_inputs(w, "categorical" if dist == 2 else "parametric", device="cuda", with_grad_out=True)
+    if rng.random() < 0.6:
+        P = np.stack([[random_pose(rng) for _ in range(n_cams)] for _ in range(batch)]).astype(np.float32)
+        x["projection_matrices"] = torch.from_numpy(P).cuda().contiguous()
+    thr = float(rng.choice([0.0, 1e-6, 1e-3]))
+    dtype = (torch.float32, torch.float16, torch.bfloat16)[int(rng.integers(0, 3))]
+    for name in ("image_feats", "depth_params"):
+        x[name] = x[name].to(dtype).contiguous()
+
+    out, cnt = U.capi_forward(x, w, dist, thr, with_count=True)
+    want, want_cnt, _ = U.oracle_forward(x, w, dist, thr, return_aux=True)
+    assert np.array_equal(cnt.cpu().numpy(), want_cnt), "per-cell sample counts differ"
+    bad, maxabs, ratio = U.violations(out.cpu().numpy(), want)
+    assert bad == 0, (bad, maxabs, ratio)
+    cache = U.capi_geometry_cache(x, w, dist)
+    got, got_cnt = U.capi_forward_cached(x, w, dist, cache, thr, with_count=True)
+    assert torch.equal(got, out) and torch.equal(got_cnt, cnt)
+    want_dd, want_df = U.oracle_backward(x, w, dist, thr)
+    for mode in ("gather", "gather_counted", "persistent_overwrite", "columns", "scatter"):
+        dd, df = U.capi_backward(x, w, dist, thr, mode=mode)
+        for got, r, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
+            bad, maxabs, ratio = U.violations(got.cpu().numpy(), r, rtol=3e-4, atol=3e-5)
+            assert bad == 0, f"seed {seed} {mode} {what}: {bad} outside tolerance (max {maxabs:.3e}, ratio {ratio:.2f})"
