@@ -104,6 +104,8 @@ struct KParams {
     unsigned cams_magic;      // i / N == umulhi(i, cams_magic) for i < 2^16
     unsigned bpb_magic;       // block / blocks_per_batch == umulhi(block, bpb_magic); 0: divide
     int gz_magic, gz_shift;   // i / gz == (i * gz_magic) >> gz_shift for 0 <= i < 4096
+    unsigned geo_lo, geo_hi;  // hash of what a geometry cache depends on besides the matrices and the sizes above it:
+                              // image size, region of interest, cell size, epsilon
 };
 
 // ---------------------------------------------------------------- element access

@@ -303,9 +303,27 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_cached_ker
     // (the cached lists are walked one group of `slots` cells at a time: their lengths are known, and
     // each cell's entries go to its own stretch of the pool)
     const int cells_per_wave = k.slots_a * k.rounds;
+    // A cache built for other sizes would send the gathers out of bounds, and one built for another region
+    // of interest or image size would pool the wrong texels: such a cache is not read at all, and the output
+    // (and the counts) are filled with NaN instead.  (The matrices themselves cannot be checked.)
+    const int *h = static_cast<const int *>(cache);
+    const bool cache_fits = h[0] == kCacheMagic && h[1] == k.B && h[2] == k.N && h[3] == k.H && h[4] == k.W && h[5] == k.gx &&
+                            h[6] == k.gy && h[7] == k.gz && h[8] == k.padded_cells && h[9] == k.NZ &&
+                            h[10] == (int)k.geo_lo && h[11] == (int)k.geo_hi;
     for (int r = 0; r < k.rounds * k.batch_groups; ++r) {
         const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots;
         if (q0 >= k.padded_cells) break;
+        if (!cache_fits) {
+            const float nan = __int_as_float(0x7fc00000);
+            for (int s = 0; s < k.slots; ++s) {
+                int ix = 0, iy = 0;
+                if (!cell_of(k, q0 + s, ix, iy)) continue;
+                const size_t cell = (size_t)((b * k.gy + iy) * k.gx + ix);
+                for (int c = lane; out != nullptr && c < k.C; c += kWave) out[cell * k.C + c] = nan;
+                if (count_out != nullptr && lane == 0) count_out[cell] = nan;
+            }
+            continue;
+        }
         phase_a_cached<T>(k, L, depth, counts, entries, b, q0, lane);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -327,10 +345,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_geometry_cache_ker
     const WaveLds L = block_lds_setup(k, smem, proj, b, 1);
     int *counts = reinterpret_cast<int *>(static_cast<char *>(cache) + kCacheHeaderBytes);
     if (blockIdx.x == 0 && threadIdx.x == 0) {
-        // what the lists were built for, for whoever inspects a cache: the library never reads it back
+        // what the lists were built for: the forward on cached geometry compares it with its own problem
         int *h = static_cast<int *>(cache);
         h[0] = kCacheMagic; h[1] = k.B; h[2] = k.N; h[3] = k.H; h[4] = k.W; h[5] = k.gx; h[6] = k.gy; h[7] = k.gz;
-        h[8] = k.padded_cells; h[9] = k.NZ;
+        h[8] = k.padded_cells; h[9] = k.NZ; h[10] = (int)k.geo_lo; h[11] = (int)k.geo_hi;
     }
     float4 *entries = reinterpret_cast<float4 *>(static_cast<char *>(cache) +
                                                  cache_entries_offset((long long)k.B * k.padded_cells));

@@ -104,6 +104,18 @@ int make_plan(const fbev_problem *p, bool allow_vec, Plan *plan, int waves = kWa
     k.xmin = p->voxel_min[0]; k.ymin = p->voxel_min[1]; k.zmin = p->voxel_min[2];
     k.vx = p->voxel_size[0]; k.vy = p->voxel_size[1]; k.vz = p->voxel_size[2];
     k.eps = p->epsilon; k.thr = p->depth_weight_threshold;
+    {
+        // FNV-1a over the bytes of the values a geometry cache was built from
+        uint64_t h = 1469598103934665603ull;
+        auto mix = [&h](const void *v, size_t n) {
+            const unsigned char *c = static_cast<const unsigned char *>(v);
+            for (size_t i = 0; i < n; ++i) h = (h ^ c[i]) * 1099511628211ull;
+        };
+        mix(&p->image_h, sizeof p->image_h); mix(&p->image_w, sizeof p->image_w);
+        mix(p->voxel_min, sizeof p->voxel_min); mix(p->voxel_size, sizeof p->voxel_size);
+        mix(&p->epsilon, sizeof p->epsilon);
+        k.geo_lo = (unsigned)h; k.geo_hi = (unsigned)(h >> 32);
+    }
     k.dist = p->depth_distribution; k.Dd = p->depth_bins;
     k.dmin = p->depth_min; k.dstep = p->depth_step;
     k.reduce_sum = p->reduction == FBEV_REDUCE_SUM;

@@ -324,8 +324,9 @@ def build_geometry_cache(projection_matrices, feature_size, image_size, roi_rang
     """Per-cell lists of the samples in view for one calibration and grid, as an opaque uint8 tensor
     for ``flash_bevpool(..., geometry_cache=...)``.  Worth building when ``projection_matrices``
     repeat from call to call (a fixed rig at inference); it must be rebuilt whenever the matrices,
-    the feature-map or image size, the grid, the region of interest or ``epsilon`` change -- nothing
-    checks that.  ``feature_size`` is (H, W) of the feature maps (a pair, or the operator's [B,N,2]
+    the feature-map or image size, the grid, the region of interest or ``epsilon`` change: a forward given
+    a cache that was built for other sizes or another region fills its output with NaN; a change of the
+    matrices alone goes unnoticed.  ``feature_size`` is (H, W) of the feature maps (a pair, or the operator's [B,N,2]
     tensor).  Size: 16 bytes per (cell, camera, height bin) sample slot."""
     ext = load_ext()
     if isinstance(feature_size, torch.Tensor):

@@ -103,8 +103,11 @@ int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, co
  * B * ceil(gx/8) * ceil(gy/8) * 64 * (4 + 16 * N * grid_z) bytes.  fbev_geometry_cache_build fills it
  * (p->channels, in_dtype and the depth fields are ignored); fbev_forward_cached is fbev_forward with
  * the cache in place of the matrices and gives the same result bit for bit.  The caller rebuilds
- * the cache whenever proj, the sizes, the grid, the region of interest or epsilon change; nothing
- * checks that.  The optional cached workspace keyed by geometry has no counterpart in the reference,
+ * the cache whenever proj, the sizes, the grid, the region of interest or epsilon change.  The cache
+ * records the sizes and a hash of image size, region of interest, cell size and epsilon; the kernel of
+ * fbev_forward_cached compares them with its own problem and, when they differ (or the memory is no
+ * cache at all), reads none of it and fills out and count_out with NaN: the call still returns
+ * FBEV_OK, since the host never reads device memory.  A change of proj alone cannot be seen.  The optional cached workspace keyed by geometry has no counterpart in the reference,
  * which recomputes the projection per channel thread (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:102-159).
  */
 size_t fbev_geometry_cache_bytes(const fbev_problem *p);

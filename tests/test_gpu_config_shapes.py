@@ -138,6 +138,19 @@ def test_cached_geometry_rejects_short_caches_and_follows_new_matrices():
     assert rc == -2
     rc = capi.geometry_cache_build(p, x["projection_matrices"].data_ptr(), cache.data_ptr(), cache.numel() - 16, 0)
     assert rc == -2
+    # a cache built for another feature-map size (same byte size: it depends on the grid and the cameras only),
+    # another region of interest or another image size is not read: NaN everywhere instead of gathers out of
+    # bounds or a silently wrong pooling
+    out = U.capi_forward(x, w, 1)
+    for other in (dataclasses.replace(w, feat_hw=(32, 88)), dataclasses.replace(w, roi_range=(-40.0, 40.0, -40.0, 40.0, -5.0, 3.0)),
+                  dataclasses.replace(w, image_hw=(512, 1408))):
+        foreign = U.capi_geometry_cache(make_inputs(other, "parametric", device="cuda"), other, 1)
+        assert foreign.numel() == cache.numel()
+        got, got_cnt = U.capi_forward_cached(x, w, 1, foreign, with_count=True)
+        assert torch.isnan(got).all() and torch.isnan(got_cnt).all()
+    garbage = torch.zeros_like(cache)
+    assert torch.isnan(U.capi_forward_cached(x, w, 1, garbage)).all()
+    assert torch.equal(U.capi_forward_cached(x, w, 1, cache), out)
     # a rebuilt cache follows the matrices it was built from
     y = dict(x, projection_matrices=x["projection_matrices"].flip(1).contiguous())
     cache2 = U.capi_geometry_cache(y, w, 1)
