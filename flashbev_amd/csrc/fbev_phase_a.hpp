@@ -327,18 +327,20 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
                                               __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
         }
         if (MODE == kModeFill && keep) {
-            // claim the sample's position in the list of its first corner texel
+            // claim the sample's position in the list of its first corner texel (compared as unsigned: counters
+            // that were not prepared for this problem may hold anything, and a negative position must not
+            // become an address)
             int pos;
             if (chunk_prefix != nullptr) {
                 // counted segments: cursor holds each segment's start within its scan chunk
                 const int i0 = tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16);
                 pos = atomicAdd(cursor + i0, 1) + chunk_prefix[i0 >> kScanChunkBits];
-                pos = pos < pair_cap ? pos : -1;
+                pos = (unsigned)pos < (unsigned)pair_cap ? pos : -1;
             } else {
                 // fixed segments of pair_cap pairs per (texel, replica): cursor counts from zero
                 const int i0 = tx.x * kFixedReplicas + (replica_of(cellxy & 0xffff, cellxy >> 16) & (kFixedReplicas - 1));
                 pos = atomicAdd(cursor + i0, 1);
-                pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
+                pos = (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
             }
             reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
         }
@@ -354,9 +356,9 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
             if (keep) {
                 if (counted) {
                     pos += chunk_prefix[i0 >> kScanChunkBits];
-                    pos = pos < pair_cap ? pos : -1;
+                    pos = (unsigned)pos < (unsigned)pair_cap ? pos : -1;
                 } else {
-                    pos = pos < pair_cap ? i0 * pair_cap + pos : -1;
+                    pos = (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
                 }
                 reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
             }
