@@ -70,7 +70,8 @@ DIST_OF = {"gaussian": (0, "parametric"), "laplace": (1, "parametric"), "categor
 class Runner:
     """Pre-allocated buffers and the four queued operations of one step."""
 
-    def __init__(self, w, depth_name: str, device: str = "cuda:0", backward_mode: int = 0, persistent: bool = True):
+    def __init__(self, w, depth_name: str, device: str = "cuda:0", backward_mode: int = 0, persistent: bool = True,
+                 sample_store: bool = True):
         self.w = w
         self.backward_mode = backward_mode
         self.dist, self.model = DIST_OF[depth_name]
@@ -85,6 +86,16 @@ class Runner:
         self.counts = torch.empty((B, gy, gx), dtype=torch.float32, device=device)
         self.vmin, self.vsize = voxel_geometry(w.roi_range, w.grid_size)
         self.eps, self.thr = 1e-6, 1e-6
+        # the sample store of a differentiated forward, where the operator would use one (small problems):
+        # the forward leaves its kept samples there and the backward's cell pass starts from them
+        self.store = None
+        if sample_store and backward_mode in (0, 2):
+            from flashbev_amd.flash_bevpool import _sample_store_limit
+            nbytes = self.ext.sample_store_bytes(x["depth_params"], x["image_feats"], x["projection_matrices"],
+                                                 x["feature_size"], x["image_size"], x["grid_size"], self.dist)
+            if 0 < nbytes <= _sample_store_limit():
+                self.store = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self.stored_by_forward = False
         # the inverse map's workspace, prepared once (what the autograd operator keeps per shape);
         # persistent=False takes a fresh workspace from the caching allocator in every call instead
         self.workspace = None
@@ -98,11 +109,13 @@ class Runner:
 
     def forward(self, cache=None):
         x, w = self.x, self.w
+        # (the forward on cached geometry leaves no samples behind: the backward then evaluates them itself)
+        self.stored_by_forward = cache is None and self.store is not None
         self.ext.flash_bevpool_forward(
             x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"], x["image_size"],
             x["grid_size"], self.vsize[0], self.vsize[1], self.vsize[2], self.vmin[0], self.vmin[1],
             self.vmin[2], self.out, self.out.numel(), self.dist, True, True, False, False, self.eps, self.thr,
-            w.depth_range[0], w.depth_range[1], 0, self.counts, cache)
+            w.depth_range[0], w.depth_range[1], 0, self.counts, cache, self.store if self.stored_by_forward else None)
 
     def geometry_cache(self):
         """Per-cell lists of the samples in view for this calibration and grid (built once)."""
@@ -117,7 +130,7 @@ class Runner:
             x["grad_out"], x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
             x["image_size"], x["roi_range"], x["grid_size"], self.d_depth, self.d_feats, self.out.numel(),
             self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0, self.backward_mode, -1,
-            self.counts, False, self.workspace)
+            self.counts, False, self.workspace, self.store if self.stored_by_forward else None)
 
 
 # Untimed steps of the workload itself, run for this many milliseconds before the warm-up steps of every

@@ -15,7 +15,7 @@ FBEV_F32, FBEV_F16, FBEV_BF16 = 0, 1, 2
 FBEV_GAUSSIAN, FBEV_LAPLACE, FBEV_CATEGORICAL = 0, 1, 2
 FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
-EXPORTS = ("fbev_forward", "fbev_geometry_cache_bytes", "fbev_geometry_cache_build", "fbev_forward_cached", "fbev_backward", "fbev_backward_gather", "fbev_backward_gather_static",
+EXPORTS = ("fbev_forward", "fbev_sample_store_bytes", "fbev_forward_store", "fbev_backward_gather_stored", "fbev_geometry_cache_bytes", "fbev_geometry_cache_build", "fbev_forward_cached", "fbev_backward", "fbev_backward_gather", "fbev_backward_gather_static",
            "fbev_static_scratch_bytes", "fbev_backward_persistent_workspace_bytes", "fbev_backward_workspace_init",
            "fbev_backward_gather_persistent", "fbev_backward_columns",
            "fbev_backward_columns_workspace_bytes", "fbev_backward_max_pairs",
@@ -56,6 +56,13 @@ def load() -> ctypes.CDLL:
         vp, pp = ctypes.c_void_p, ctypes.POINTER(FbevProblem)
         lib.fbev_forward.argtypes = [pp, vp, vp, vp, vp, vp, vp]
         lib.fbev_forward.restype = ctypes.c_int
+        lib.fbev_sample_store_bytes.argtypes = [pp]
+        lib.fbev_sample_store_bytes.restype = ctypes.c_size_t
+        lib.fbev_forward_store.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp]
+        lib.fbev_forward_store.restype = ctypes.c_int
+        lib.fbev_backward_gather_stored.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp, vp, ctypes.c_int, vp,
+                                                    ctypes.c_size_t, ctypes.c_int, vp]
+        lib.fbev_backward_gather_stored.restype = ctypes.c_int
         lib.fbev_geometry_cache_bytes.argtypes = [pp]
         lib.fbev_geometry_cache_bytes.restype = ctypes.c_size_t
         lib.fbev_geometry_cache_build.argtypes = [pp, vp, vp, ctypes.c_size_t, vp]
@@ -149,6 +156,29 @@ def forward(p: FbevProblem, depth_ptr: int, feats_ptr: int, proj_ptr: int, out_p
             stream: int = 0, count_ptr: Optional[int] = None) -> int:
     return load().fbev_forward(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(proj_ptr), _p(out_ptr),
                                _p(count_ptr), _p(stream))
+
+
+def sample_store_bytes(p: FbevProblem) -> int:
+    return int(load().fbev_sample_store_bytes(ctypes.byref(p)))
+
+
+def forward_store(p: FbevProblem, depth_ptr: int, feats_ptr: int, proj_ptr: int, out_ptr: int, count_out_ptr: int,
+                  store_ptr: int, store_bytes: int, stream: int = 0) -> int:
+    """fbev_forward that also leaves the kept samples' records in `store` for backward_gather_stored."""
+    return load().fbev_forward_store(ctypes.byref(p), _p(depth_ptr), _p(feats_ptr), _p(proj_ptr), _p(out_ptr),
+                                     _p(count_out_ptr), _p(store_ptr), ctypes.c_size_t(int(store_bytes)), _p(stream))
+
+
+def backward_gather_stored(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
+                           cell_count_ptr: int, store_ptr: int, store_bytes: int, d_depth_ptr: Optional[int],
+                           d_feats_ptr: Optional[int], workspace_ptr: int, workspace_bytes: int, stream: int = 0,
+                           accumulate: bool = True, persistent: bool = False) -> int:
+    """fbev_backward_gather(_persistent) whose cell pass starts from the records forward_store left."""
+    return load().fbev_backward_gather_stored(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
+                                              _p(proj_ptr), _p(cell_count_ptr), _p(store_ptr),
+                                              ctypes.c_size_t(int(store_bytes)), _p(d_depth_ptr), _p(d_feats_ptr),
+                                              int(bool(accumulate)), _p(workspace_ptr),
+                                              ctypes.c_size_t(int(workspace_bytes)), int(bool(persistent)), _p(stream))
 
 
 def geometry_cache_bytes(p: FbevProblem) -> int:

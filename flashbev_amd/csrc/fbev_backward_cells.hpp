@@ -156,7 +156,9 @@ __global__ __launch_bounds__(1024) void fbev_scan_sums_kernel(int *v, int n) {
 }
 
 // Cell pass of the backward.  FILL = 0: scatter with atomics.  FILL = 1: write pairs (inverse
-// map); FILL = 2: the same with one claim per run of samples on one texel.
+// map); FILL = 2: the same with one claim per run of samples on one texel; FILL = 3: write pairs for the
+// samples the forward stored (`store`, with the forward's per-cell counts in `count`) instead of
+// evaluating the samples again.
 // `cursor` holds, on entry, the start (within its scan chunk) of every (texel, replica)
 // segment; phase A advances it, so on exit cursor[i] is the END of segment i.
 template <typename T, int VEC, int CPL, int FILL, bool BATCHED>
@@ -164,9 +166,11 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     KParams k, const float *__restrict__ grad_out, const T *__restrict__ depth, const T *__restrict__ feats,
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
     const int *__restrict__ chunk_prefix, int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap,
-    int *epoch, int set_stride) {
+    int *epoch, int set_stride, const float *__restrict__ count = nullptr, const float4 *__restrict__ store = nullptr) {
     extern __shared__ float4 smem[];
     constexpr int EF4 = 2;
+    constexpr bool STORED = FILL == 3;
+    static_assert(!(STORED && BATCHED), "the stored samples of a batch go through in one piece");
     if (FILL && epoch != nullptr) {
         // persistent workspace: the call counter's low bit selects the set of claim counters, and the
         // texel pass finds the counter where no block of its own writes (see struct Persist)
@@ -183,7 +187,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     const int b = batch_of(k, bid);
     const int blk = bid - b * k.blocks_per_batch;
 
-    const WaveLds L = block_lds_setup(k, smem, proj, b, EF4);
+    // (nothing is projected when the samples come from the store: no matrices, no tables)
+    const WaveLds L = STORED ? wave_lds_view(k, smem, EF4) : block_lds_setup(k, smem, proj, b, EF4);
     lds_counter *cnt = L.cnt;
     float4 *lst = L.lst;
 
@@ -252,7 +257,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
         };
         enter_group(0);
         load_g(0);
-        const int n_cand = phase_a_candidates<BATCHED>(k, L, q0, lane);
+        const int n_cand = STORED ? 0 : phase_a_candidates<BATCHED>(k, L, q0, lane);
         // all groups of the batch through stage 2 together when the pool is sure to hold what they keep
         const int n_groups = BATCHED ? k.batch_groups : 1;
         const int step = n_cand <= k.pool_cap ? n_groups : 1;
@@ -261,9 +266,13 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
             enter_group(g0);
             load_g(0);
         }
-        phase_a_samples<EF4, T, FILL == 2 ? kModeFillRuns : (FILL ? kModeFill : kModeScatter)>(
-            k, L, depth, b, lane, BATCHED ? L.gcand[g0] : 0, BATCHED ? L.gcand[g0 + step] : n_cand, chunk_prefix, cursor,
-            pair_cap);
+        if (STORED)
+            phase_a_stored(k, L, count, store + ((size_t)b * k.padded_cells + q0) * k.NZ * 2, b, q0, lane, chunk_prefix,
+                           cursor, pair_cap);
+        else
+            phase_a_samples<EF4, T, FILL == 2 ? kModeFillRuns : (FILL ? kModeFill : kModeScatter)>(
+                k, L, depth, b, lane, BATCHED ? L.gcand[g0] : 0, BATCHED ? L.gcand[g0 + step] : n_cand, chunk_prefix, cursor,
+                pair_cap);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         for (int grp = g0; grp < g0 + step; ++grp) {
@@ -308,6 +317,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                 const bool spill = FILL ? __float_as_int(geo.w) < 0 : true;
                 const bool s00 = spill, s01 = spill, s10 = spill, s11 = spill;
                 const float a00 = w00 * wgt, a01 = w01 * wgt, a10 = w10 * wgt, a11 = w11 * wgt;
+                // <grad_out, sampled feature> = sum over the corners of w_ij * <grad_out, row_ij>: the four inner
+                // products take the rows as they come (half-precision rows enter the multiply-adds unconverted),
+                // and the bilinear weights are applied once per entry instead of once per channel
+                float d00 = 0.0f, d01 = 0.0f, d10 = 0.0f, d11 = 0.0f;
 #pragma unroll
                 for (int j = 0; j < CPL; ++j) {
                     const int ch = c0 + (j * k.lanes_per_slot + lis) * VEC;
@@ -321,9 +334,10 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                             VecLoad<T, VEC>::ld(row_at(r11 + chb), f11);
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) {
-                                const float f = __builtin_fmaf(w11, f11[v], __builtin_fmaf(w10, f10[v],
-                                                __builtin_fmaf(w01, f01[v], w00 * f00[v])));
-                                G = __builtin_fmaf(g[j][v], f, G);
+                                d00 = __builtin_fmaf(g[j][v], f00[v], d00);
+                                d01 = __builtin_fmaf(g[j][v], f01[v], d01);
+                                d10 = __builtin_fmaf(g[j][v], f10[v], d10);
+                                d11 = __builtin_fmaf(g[j][v], f11[v], d11);
                             }
                         }
                         if (d_feats != nullptr && (s00 || s01 || s10 || s11)) {
@@ -339,6 +353,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
                         }
                     }
                 }
+                if (need_G) G = __builtin_fmaf(w11, d11, __builtin_fmaf(w10, d10, __builtin_fmaf(w01, d01, w00 * d00)));
                 return G;
             };
             // what one lane does with the complete G of entry e

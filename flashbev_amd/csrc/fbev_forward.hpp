@@ -159,10 +159,12 @@ __device__ __forceinline__ void forward_phase_b(const KParams &k, const WaveLds 
     }
 }
 
-template <typename T, int VEC, int CPL, bool STREAM, bool BATCHED>
+// STORE: the forward of a call that will be differentiated also leaves every kept sample's record in
+// `store` (see kModeForwardStore), so that the backward's cell pass need not evaluate the samples again.
+template <typename T, int VEC, int CPL, bool STREAM, bool BATCHED, bool STORE = false>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
     KParams k, const T *__restrict__ depth, const T *__restrict__ feats, const float *__restrict__ proj,
-    float *__restrict__ out, float *__restrict__ count_out) {
+    float *__restrict__ out, float *__restrict__ count_out, float4 *__restrict__ store = nullptr) {
     extern __shared__ float4 smem[];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -181,8 +183,9 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_forward_kernel(
         const int n_groups = BATCHED ? k.batch_groups : 1;
         const int step = n_cand <= k.pool_cap ? n_groups : 1;
         for (int g = 0; g < n_groups; g += step) {
-            phase_a_samples<2, T, kModeForward>(k, L, depth, b, lane, BATCHED ? L.gcand[g] : 0,
-                                                BATCHED ? L.gcand[g + step] : n_cand);
+            phase_a_samples<2, T, STORE ? kModeForwardStore : kModeForward>(
+                k, L, depth, b, lane, BATCHED ? L.gcand[g] : 0, BATCHED ? L.gcand[g + step] : n_cand, nullptr, nullptr, 0,
+                STORE ? store + ((size_t)b * k.padded_cells + q0) * k.NZ * 2 : nullptr);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             for (int j = g; j < g + step; ++j) forward_phase_b<T, VEC, CPL, STREAM>(k, L, role, b, j, feats, out, count_out);

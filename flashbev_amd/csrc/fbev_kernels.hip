@@ -232,15 +232,16 @@ bool lds_opt_in(Kernel kernel, size_t lds) {
 
 template <typename T, int VEC>
 int launch_forward(const Plan &pl, const void *depth, const void *feats, const float *proj, float *out,
-                   float *cnt, hipStream_t st) {
+                   float *cnt, hipStream_t st, float4 *store = nullptr) {
     dim3 grid(pl.k.n_blocks), block(kWave * pl.k.waves);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
     prof::Scope timer(out != nullptr ? prof::kForward : prof::kCellCount, st);
-    const bool stream = VEC > 1 && (long long)pl.k.B * pl.k.gy * pl.k.gx * pl.k.C * 4 > kStreamOutputFrom;
+    // (a forward that stores its samples writes its output with ordinary stores: the problems it serves are small)
+    const bool stream = store == nullptr && VEC > 1 && (long long)pl.k.B * pl.k.gy * pl.k.gx * pl.k.C * 4 > kStreamOutputFrom;
     auto launch = [&](auto kernel) {
         if (!lds_opt_in(kernel, pl.lds_fwd)) return false;
-        hipLaunchKernelGGL(kernel, grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt);
+        hipLaunchKernelGGL(kernel, grid, block, pl.lds_fwd, st, pl.k, d, f, proj, out, cnt, store);
         return true;
     };
     // (batches of several groups and streamed output exist on the vector paths only; the plan asks for
@@ -250,6 +251,8 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
     if (!V && pl.k.batch_groups > 1) return FBEV_ERR_LAUNCH;
     auto pick = [&](auto cpl_tag) {
         constexpr int CPL = decltype(cpl_tag)::value;
+        if (store != nullptr)
+            return batched ? launch(fbev_forward_kernel<T, VEC, CPL, false, V, true>) : launch(fbev_forward_kernel<T, VEC, CPL, false, false, true>);
         if (stream) return batched ? launch(fbev_forward_kernel<T, VEC, CPL, V, V>) : launch(fbev_forward_kernel<T, VEC, CPL, V, false>);
         return batched ? launch(fbev_forward_kernel<T, VEC, CPL, false, V>) : launch(fbev_forward_kernel<T, VEC, CPL, false, false>);
     };
@@ -260,18 +263,26 @@ int launch_forward(const Plan &pl, const void *depth, const void *feats, const f
 }
 
 int dispatch_forward(const fbev_problem *p, const Plan &pl, const void *depth, const void *feats, const float *proj,
-                     float *out, float *cnt, hipStream_t st) {
+                     float *out, float *cnt, hipStream_t st, float4 *store = nullptr) {
     switch (p->in_dtype) {
         case FBEV_F32:
-            return pl.vec == 4 ? launch_forward<float, 4>(pl, depth, feats, proj, out, cnt, st)
-                               : launch_forward<float, 1>(pl, depth, feats, proj, out, cnt, st);
+            return pl.vec == 4 ? launch_forward<float, 4>(pl, depth, feats, proj, out, cnt, st, store)
+                               : launch_forward<float, 1>(pl, depth, feats, proj, out, cnt, st, store);
         case FBEV_F16:
-            return pl.vec == 8 ? launch_forward<__half, 8>(pl, depth, feats, proj, out, cnt, st)
-                               : launch_forward<__half, 1>(pl, depth, feats, proj, out, cnt, st);
+            return pl.vec == 8 ? launch_forward<__half, 8>(pl, depth, feats, proj, out, cnt, st, store)
+                               : launch_forward<__half, 1>(pl, depth, feats, proj, out, cnt, st, store);
         default:
-            return pl.vec == 8 ? launch_forward<bf16_raw, 8>(pl, depth, feats, proj, out, cnt, st)
-                               : launch_forward<bf16_raw, 1>(pl, depth, feats, proj, out, cnt, st);
+            return pl.vec == 8 ? launch_forward<bf16_raw, 8>(pl, depth, feats, proj, out, cnt, st, store)
+                               : launch_forward<bf16_raw, 1>(pl, depth, feats, proj, out, cnt, st, store);
     }
+}
+
+// Bytes of a sample store: per cell of the tiled walk a slot of N * gz records of 32 bytes.
+size_t sample_store_bytes(const fbev_problem *p) {
+    const long long tiles = (long long)((p->grid_x + kTile - 1) / kTile) * ((p->grid_y + kTile - 1) / kTile);
+    // a stored first-corner texel shares its word with the two clamp flags
+    if ((long long)p->batch * p->num_cams * p->feat_h * p->feat_w >= (1ll << 29)) return 0;
+    return (size_t)p->batch * (size_t)tiles * 64 * (size_t)p->num_cams * (size_t)p->grid_z * 2 * sizeof(float4);
 }
 
 template <typename T, int VEC>
@@ -325,7 +336,7 @@ int launch_columns(const Plan &pl, const ColParams &cp, size_t lds, const float 
 template <typename T, int VEC, int FILL>
 int launch_cells(const Plan &pl, const float *go, const void *depth, const void *feats, const float *proj,
                  float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap, hipStream_t st,
-                 int *epoch = nullptr, int set_stride = 0) {
+                 int *epoch = nullptr, int set_stride = 0, const float *count = nullptr, const float4 *store = nullptr) {
     dim3 grid(pl.k.n_blocks), block(kWave * pl.k.waves);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
@@ -336,12 +347,18 @@ int launch_cells(const Plan &pl, const float *go, const void *depth, const void 
     if (!V && pl.k.batch_groups > 1) return FBEV_ERR_LAUNCH;
     auto launch = [&](auto kernel) {
         if (!lds_opt_in(kernel, lds)) return false;
-        hipLaunchKernelGGL(kernel, grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride);
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride,
+                           count, store);
         return true;
     };
     auto pick = [&](auto cpl_tag) {
         constexpr int CPL = decltype(cpl_tag)::value;
-        return batched ? launch(fbev_backward_cells_kernel<T, VEC, CPL, FILL, V>) : launch(fbev_backward_cells_kernel<T, VEC, CPL, FILL, false>);
+        if constexpr (FILL == 3) {
+            // stored samples go through a batch in one piece: the plan has one group per batch
+            return !batched && launch(fbev_backward_cells_kernel<T, VEC, CPL, FILL, false>);
+        } else {
+            return batched ? launch(fbev_backward_cells_kernel<T, VEC, CPL, FILL, V>) : launch(fbev_backward_cells_kernel<T, VEC, CPL, FILL, false>);
+        }
     };
     const bool ok = pl.cpl == 1 ? pick(std::integral_constant<int, 1>{})
                                 : (pl.cpl == 2 ? pick(std::integral_constant<int, 2>{}) : pick(std::integral_constant<int, 4>{}));
@@ -392,17 +409,18 @@ bool cells_batch_pays(const fbev_problem *p, const Plan &pl) {
 template <int FILL>
 int dispatch_cells(const fbev_problem *p, const Plan &pl, const float *go, const void *depth, const void *feats,
                    const float *proj, float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap,
-                   hipStream_t st, int *epoch = nullptr, int set_stride = 0) {
+                   hipStream_t st, int *epoch = nullptr, int set_stride = 0, const float *count = nullptr,
+                   const float4 *store = nullptr) {
     switch (p->in_dtype) {
         case FBEV_F32:
-            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride)
-                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride);
+            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store)
+                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store);
         case FBEV_F16:
-            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride)
-                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride);
+            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store)
+                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store);
         default:
-            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride)
-                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride);
+            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store)
+                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store);
     }
 }
 
@@ -502,7 +520,8 @@ int scratch_of_current_device(void **out) {
 
 int backward_gather_impl(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
                          const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
-                         size_t workspace_bytes, void *stream, bool persistent = false) {
+                         size_t workspace_bytes, void *stream, bool persistent = false, const float *cell_count = nullptr,
+                         const void *store = nullptr, size_t store_bytes = 0) {
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
     rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
@@ -523,9 +542,25 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     const int cap = cap64 > 0x7fffffffull ? 0x7fffffff : (int)cap64;
     Plan pl;
     const bool allow_vec = (uintptr_t)feats % 16 == 0 && (uintptr_t)grad_out % 16 == 0;
-    rc = make_plan(p, allow_vec, &pl, kCellPassWaves);
+    // the samples the forward stored serve where claims are made one by one (the only kind phase_a_stored makes)
+    bool stored = store != nullptr;
+    if (stored) {
+        // (where a claim counter may get hundreds of samples the claims go per run, which the stored samples do
+        // not: such problems evaluate their samples again)
+        const long long tx = texel_count(p);
+        const bool fixed_layout = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (tx * kFixedReplicas) >= kFixedMinSegment;
+        if (sample_count(p) / (fixed_layout ? tx * kFixedReplicas : counter_count(p)) >= kClaimRunsFrom) stored = false;
+    }
+    if (stored) {
+        if (!cell_count) return FBEV_ERR_NULL;
+        if ((uintptr_t)store % 16 || (uintptr_t)cell_count % 4) return FBEV_ERR_ALIGNMENT;
+        const size_t need = sample_store_bytes(p);
+        if (need == 0) return FBEV_ERR_TOO_LARGE;
+        if (store_bytes < need) return FBEV_ERR_SHAPE;
+    }
+    rc = make_plan(p, allow_vec, &pl, kCellPassWaves, 3, kMaxSlotLdsBytes, stored ? 1 : 4);
     if (rc != FBEV_OK) return rc;
-    {
+    if (!stored) {
         // the cell pass in batches of several groups only where that does not cost occupancy
         const long long tx = texel_count(p);
         const bool fixed_layout = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (tx * kFixedReplicas) >= kFixedMinSegment;
@@ -590,6 +625,10 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     const int cap_arg = fixed ? seg_cap : cap;
     // samples a claim counter gets if every sample is kept
     const bool claim_runs = sample_count(p) / (fixed ? texels * kFixedReplicas : counters) >= kClaimRunsFrom;
+    if (stored)
+        rc = dispatch_cells<3>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs, cap_arg, st,
+                               ps.epoch, ps.set_stride, cell_count, static_cast<const float4 *>(store));
+    else
     rc = claim_runs ? dispatch_cells<2>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs,
                                         cap_arg, st, ps.epoch, ps.set_stride)
                     : dispatch_cells<1>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs,
@@ -672,6 +711,30 @@ int fbev_forward(const fbev_problem *p, const void *depth, const void *feats, co
     rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kCellPassWaves, 4);
     if (rc != FBEV_OK) return rc;
     return dispatch_forward(p, pl, depth, feats, proj, out, count_out, static_cast<hipStream_t>(stream));
+}
+
+size_t fbev_sample_store_bytes(const fbev_problem *p) {
+    if (validate(p, true) != FBEV_OK) return 0;
+    return sample_store_bytes(p);
+}
+
+int fbev_forward_store(const fbev_problem *p, const void *depth, const void *feats, const float *proj, float *out,
+                       float *count_out, void *store, size_t store_bytes, void *stream) {
+    int rc = validate(p, true);
+    if (rc != FBEV_OK) return rc;
+    if (!depth || !feats || !proj || !out || !count_out || !store) return FBEV_ERR_NULL;
+    const int es = elem_size(p->in_dtype);
+    if ((uintptr_t)depth % es || (uintptr_t)feats % es || (uintptr_t)proj % 4 || (uintptr_t)out % 4 ||
+        (uintptr_t)count_out % 4 || (uintptr_t)store % 16)
+        return FBEV_ERR_ALIGNMENT;
+    const size_t need = sample_store_bytes(p);
+    if (need == 0) return FBEV_ERR_TOO_LARGE;
+    if (store_bytes < need) return FBEV_ERR_SHAPE;
+    Plan pl;
+    rc = make_plan(p, (uintptr_t)feats % 16 == 0 && (uintptr_t)out % 16 == 0, &pl, kCellPassWaves, 4);
+    if (rc != FBEV_OK) return rc;
+    return dispatch_forward(p, pl, depth, feats, proj, out, count_out, static_cast<hipStream_t>(stream),
+                            static_cast<float4 *>(store));
 }
 
 size_t fbev_geometry_cache_bytes(const fbev_problem *p) {
@@ -841,6 +904,15 @@ int fbev_backward_gather_persistent(const fbev_problem *p, const float *grad_out
                                     size_t workspace_bytes, void *stream) {
     return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
                                 workspace_bytes, stream, true);
+}
+
+int fbev_backward_gather_stored(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                                const float *proj, const float *cell_count, const void *store, size_t store_bytes,
+                                float *d_depth, float *d_feats, int accumulate, void *workspace, size_t workspace_bytes,
+                                int persistent, void *stream) {
+    if (!store) return FBEV_ERR_NULL;
+    return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
+                                workspace_bytes, stream, persistent != 0, cell_count, store, store_bytes);
 }
 
 int fbev_backward_gather_static(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,

@@ -93,7 +93,30 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 //                     the two flags below it, and in the fourth place the position of the sample's
 //                     pair in the pair array (sorted by first corner texel), or -1 if the array is full
 //             word 1: wgt, a, b, (k0 | k1 << 16)
-enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeFillRuns = 4, kModeCache = 5 };
+//   store     what a forward that is going to be differentiated leaves behind for the backward's cell pass, two
+//             words per kept sample in the slot of its cell (cells in the order of the tiled walk, N * gz entries
+//             per cell): the backward entry above with -1 in the fourth place (no pair position yet)
+enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeFillRuns = 4, kModeCache = 5,
+       kModeForwardStore = 6 };
+
+// Position of a kept sample's pair in the list of its first corner texel: one returning integer atomic
+// on the counter the sample's cell selects among the texel's replicas.  -1: the list is full (compared
+// as unsigned: counters that were not prepared for this problem may hold anything, and a negative
+// position must not become an address).
+__device__ __forceinline__ int claim_pair(const int *__restrict__ chunk_prefix, int *__restrict__ cursor, int pair_cap,
+                                          int texel, int cellxy) {
+    const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
+    if (chunk_prefix != nullptr) {
+        // counted segments: cursor holds each segment's start within its scan chunk
+        const int i0 = texel * kReplicas + rep;
+        const int pos = atomicAdd(cursor + i0, 1) + chunk_prefix[i0 >> kScanChunkBits];
+        return (unsigned)pos < (unsigned)pair_cap ? pos : -1;
+    }
+    // fixed segments of pair_cap pairs per (texel, replica): cursor counts from zero
+    const int i0 = texel * kFixedReplicas + (rep & (kFixedReplicas - 1));
+    const int pos = atomicAdd(cursor + i0, 1);
+    return (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
+}
 
 // Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
 // pixel coordinate misses the image by more than this fraction, far beyond any rounding of
@@ -224,9 +247,11 @@ template <int ENTRY_F4, typename T, int MODE>
 __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds &L, const T *__restrict__ depth, int b,
                                                 int lane, int c_lo, int c_hi,
                                                 const int *__restrict__ chunk_prefix = nullptr,
-                                                int *__restrict__ cursor = nullptr, int pair_cap = 0) {
+                                                int *__restrict__ cursor = nullptr, int pair_cap = 0,
+                                                float4 *__restrict__ store = nullptr) {
     constexpr bool FILLING = MODE == kModeFill || MODE == kModeFillRuns;   // the latter claims per run
     constexpr bool BACKWARD = MODE == kModeScatter || FILLING;
+    constexpr bool STORING = MODE == kModeForwardStore;      // `store`: the slot of the batch's first cell
     if (lane < k.slots_a) L.cnt[lane] = 0;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -239,7 +264,7 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
         const int d = __float_as_int(col.w);
         const int slot = active ? (d >> 28) & 15 : 16 + (lane & 1);   // idle lanes: no real cell
         const int cam = (d >> 16) & 0xfff;
-        float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w2 = w0;
+        float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w2 = w0, rec = w0;
         int4 tx = make_int4(0, 0, 0, 0);
         int cellxy = 0;
         bool keep = false;
@@ -279,6 +304,11 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
                 w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
             } else {
                 w0 = make_float4(w00 * e.wgt, w01 * e.wgt, w10 * e.wgt, w11 * e.wgt);
+                if (STORING) {
+                    const int fl = (g.u1 != g.u0 ? 1 : 0) | (g.v1 != g.v0 ? 2 : 0);
+                    rec = make_float4(g.du, g.dv, __int_as_float((t00 << 2) | fl), __int_as_float(-1));
+                    w2 = make_float4(e.wgt, e.a, e.b, __int_as_float(e.k0 | (e.k1 << 16)));
+                }
             }
         }
         const int prev_slot = __shfl_up(slot, 1, kWave);
@@ -326,24 +356,14 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
                                 : make_float4(__int_as_float(tx.x * k.row_units), __int_as_float(tx.y * k.row_units),
                                               __int_as_float(tx.z * k.row_units), __int_as_float(tx.w * k.row_units));
         }
-        if (MODE == kModeFill && keep) {
-            // claim the sample's position in the list of its first corner texel (compared as unsigned: counters
-            // that were not prepared for this problem may hold anything, and a negative position must not
-            // become an address)
-            int pos;
-            if (chunk_prefix != nullptr) {
-                // counted segments: cursor holds each segment's start within its scan chunk
-                const int i0 = tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16);
-                pos = atomicAdd(cursor + i0, 1) + chunk_prefix[i0 >> kScanChunkBits];
-                pos = (unsigned)pos < (unsigned)pair_cap ? pos : -1;
-            } else {
-                // fixed segments of pair_cap pairs per (texel, replica): cursor counts from zero
-                const int i0 = tx.x * kFixedReplicas + (replica_of(cellxy & 0xffff, cellxy >> 16) & (kFixedReplicas - 1));
-                pos = atomicAdd(cursor + i0, 1);
-                pos = (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
-            }
-            reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
+        if (STORING && keep) {
+            // the sample's record for the backward, at its place among the kept samples of its cell
+            float4 *dst = store + ((size_t)slot * k.NZ + old + __popcll(m & seg & lanemask_lt(lane))) * 2;
+            dst[0] = rec;
+            dst[1] = w2;
         }
+        if (MODE == kModeFill && keep)
+            reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = claim_pair(chunk_prefix, cursor, pair_cap, tx.x, cellxy);
         if (MODE == kModeFillRuns) {
             // the same, but the run's first lane claims for the whole run (same cell and texel: same
             // counter) and hands the positions out; every lane takes part in the exchange
@@ -368,6 +388,60 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
             // when these are its first, where they start in the pool (a cell without entries has no start)
             L.cnt[slot] = old + __popcll(m & seg);
             if (old == 0) L.start[slot] = at;
+        }
+    }
+}
+
+// The sample phase of the backward's cell pass when the forward left its kept samples behind (kModeForwardStore):
+// lanes = the stored samples of the batch's cells, densely packed; each is copied into the pool and claims
+// its pair position.  No matrices, no projection, no depth model.  `count` holds the forward's per-cell
+// counts, [B, gy, gx]; `store` points at the slot of the batch's first cell.  Values that cannot have come
+// from a forward of this problem (a count beyond N * gz, a texel beyond the feature maps) are clamped and
+// zeroed, so that a wrong buffer gives wrong numbers but no access out of bounds.
+__device__ __forceinline__ void phase_a_stored(const KParams &k, const WaveLds &L, const float *__restrict__ count,
+                                               const float4 *__restrict__ store, int b, int q0, int lane,
+                                               const int *__restrict__ chunk_prefix, int *__restrict__ cursor,
+                                               int pair_cap) {
+    int mine_n = 0, mine_xy = 0;
+    if (lane < k.slots_a) {
+        int ix = 0, iy = 0;
+        if (cell_of(k, q0 + lane, ix, iy)) {
+            mine_n = min(max((int)count[(size_t)(b * k.gy + iy) * k.gx + ix], 0), k.NZ);
+            mine_xy = ix | (iy << 16);
+        }
+    }
+    int incl = mine_n;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        const int other = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += other;
+    }
+    const int total = __shfl(incl, 15, kWave);        // slots_a <= 16; lanes past the cells carry 0
+    const int my_start = incl - mine_n;
+    if (lane < k.slots_a) {
+        L.cnt[lane] = mine_n;
+        L.start[lane] = my_start;
+    }
+    const unsigned n_texels = (unsigned)(k.B * k.N * k.H * k.W);
+    for (int jb = 0; jb < total; jb += kWave) {
+        const int j = jb + lane;
+        // the cell whose stretch holds j: the last one that starts at or before j (empty cells start
+        // where the next one does, so later ones win)
+        int slot = 0;
+        for (int s = 1; s < k.slots_a; ++s) slot = (__shfl(my_start, s, kWave) <= j) ? s : slot;
+        const int first = __shfl(my_start, slot, kWave);
+        const int cellxy = __shfl(mine_xy, slot, kWave);
+        if (j < total) {
+            // (only cells of the walk have a count above zero, so the slot exists)
+            const float4 *src = store + ((size_t)slot * k.NZ + (j - first)) * 2;
+            float4 geo = src[0], dw = src[1];
+            if ((unsigned)(__float_as_int(geo.z) >> 2) >= n_texels) {
+                geo = make_float4(0.f, 0.f, __int_as_float(0), 0.f);
+                dw = make_float4(0.f, 0.f, 0.f, __int_as_float(1 << 16));
+            }
+            geo.w = __int_as_float(claim_pair(chunk_prefix, cursor, pair_cap, __float_as_int(geo.z) >> 2, cellxy));
+            L.lst[2 * j] = geo;
+            L.lst[2 * j + 1] = dw;
         }
     }
 }

@@ -163,7 +163,7 @@ void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &ima
                            bool use_shared_memory, bool optimize_z_precompute, bool use_warp_kernel,
                            bool use_vectorized_load, float epsilon, float depth_weight_threshold,
                            float depth_min, float depth_step, int reduction, std::optional<at::Tensor> count_out,
-                           std::optional<at::Tensor> geometry_cache) {
+                           std::optional<at::Tensor> geometry_cache, std::optional<at::Tensor> sample_store) {
     (void)use_shared_memory; (void)optimize_z_precompute; (void)use_warp_kernel; (void)use_vectorized_load;
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
@@ -195,9 +195,28 @@ void flash_bevpool_forward(const at::Tensor &depth_params, const at::Tensor &ima
                  "fbev_forward_cached");
         return;
     }
+    if (sample_store.has_value() && sample_store->defined()) {
+        // a forward that will be differentiated: the kept samples' records stay behind for flash_bevpool_backward
+        check_dev(*sample_store, depth_params, "sample_store");
+        TORCH_CHECK(sample_store->scalar_type() == at::kByte, "flashbevpool_ext: sample_store must be a uint8 tensor");
+        TORCH_CHECK(cnt != nullptr, "flashbevpool_ext: sample_store needs count_out");
+        raise_on(fbev_forward_store(&p, depth_params.data_ptr(), image_feats.data_ptr(), projection_matrices.data_ptr<float>(),
+                                    out.data_ptr<float>(), cnt, sample_store->data_ptr(), (size_t)sample_store->numel(), st),
+                 "fbev_forward_store");
+        return;
+    }
     raise_on(fbev_forward(&p, depth_params.data_ptr(), image_feats.data_ptr(), projection_matrices.data_ptr<float>(),
                           out.data_ptr<float>(), cnt, st),
              "fbev_forward");
+}
+
+// Bytes of the sample store flash_bevpool_forward(..., sample_store=...) fills for these tensors (0: none).
+int64_t sample_store_bytes(const at::Tensor &depth_params, const at::Tensor &image_feats,
+                           const at::Tensor &projection_matrices, const at::Tensor &feature_size,
+                           const at::Tensor &image_size, const at::Tensor &grid_size, int depth_distribution) {
+    fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              depth_distribution, 1e-6f, 0.0f, 1.0f, 1.0f, 0);
+    return (int64_t)fbev_sample_store_bytes(&p);
 }
 
 // The per-cell lists of samples in view for these matrices and this grid (fbev_geometry_cache_build),
@@ -243,7 +262,7 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                             int64_t total_threads, int depth_distribution, float epsilon, float depth_weight_threshold,
                             float depth_min, float depth_step, int reduction, int backward_mode,
                             int64_t pair_capacity, std::optional<at::Tensor> cell_count, bool accumulate,
-                            std::optional<at::Tensor> workspace) {
+                            std::optional<at::Tensor> workspace, std::optional<at::Tensor> sample_store) {
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
     auto roi = host_floats(roi_range, 6, "roi_range");
@@ -278,6 +297,23 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
     TORCH_CHECK(backward_mode >= 0 && backward_mode <= 3,
                 "flashbevpool_ext: backward_mode must be 0 (auto), 1 (atomic scatter), 2 (inverse-map gather) or "
                 "3 (column owner)");
+    // the records and counts the forward left (flash_bevpool_forward(..., count_out, sample_store)), if any
+    const float *stored_count = nullptr;
+    const void *store = nullptr;
+    size_t store_bytes = 0;
+    if (sample_store.has_value() && sample_store->defined()) {
+        check_dev(*sample_store, depth_params, "sample_store");
+        TORCH_CHECK(sample_store->scalar_type() == at::kByte, "flashbevpool_ext: sample_store must be a uint8 tensor");
+        TORCH_CHECK(cell_count.has_value() && cell_count->defined(), "flashbevpool_ext: sample_store needs cell_count");
+        check_dev(*cell_count, depth_params, "cell_count");
+        TORCH_CHECK(cell_count->scalar_type() == at::kFloat && cell_count->numel() == (int64_t)p.batch * p.grid_y * p.grid_x,
+                    "flashbevpool_ext: cell_count must be float32 [B,grid_y,grid_x]");
+        TORCH_CHECK(backward_mode == 0 || backward_mode == 2,
+                    "flashbevpool_ext: a sample store goes with backward_mode 0 (auto) or 2 (gather)");
+        stored_count = cell_count->data_ptr<float>();
+        store = sample_store->data_ptr();
+        store_bytes = (size_t)sample_store->numel();
+    }
     auto run_columns = [&]() -> int {
         const float *cnt = nullptr;
         at::Tensor ws;
@@ -310,6 +346,10 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
         if (cap > max_pairs) cap = max_pairs;
         const size_t bytes = fbev_backward_workspace_bytes(&p, cap);
         at::Tensor ws = at::empty({(int64_t)bytes}, at::TensorOptions().device(depth_params.device()).dtype(at::kByte));
+        if (store != nullptr)
+            return fbev_backward_gather_stored(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                                               projection_matrices.data_ptr<float>(), stored_count, store, store_bytes, dd, df,
+                                               accumulate ? 1 : 0, ws.data_ptr(), bytes, 0, st);
         return fbev_backward_gather(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
                                     projection_matrices.data_ptr<float>(), dd, df, accumulate ? 1 : 0, ws.data_ptr(),
                                     bytes, st);
@@ -320,10 +360,16 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                     "flashbevpool_ext: a persistent workspace goes with backward_mode 0 (auto) or 2 (gather)");
         check_dev(*workspace, depth_params, "workspace");
         TORCH_CHECK(workspace->scalar_type() == at::kByte, "flashbevpool_ext: workspace must be a uint8 tensor");
-        raise_on(fbev_backward_gather_persistent(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(),
-                                                 image_feats.data_ptr(), projection_matrices.data_ptr<float>(), dd, df,
-                                                 accumulate ? 1 : 0, workspace->data_ptr(), (size_t)workspace->numel(), st),
-                 "fbev_backward_gather_persistent");
+        if (store != nullptr)
+            raise_on(fbev_backward_gather_stored(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                                                 projection_matrices.data_ptr<float>(), stored_count, store, store_bytes, dd, df,
+                                                 accumulate ? 1 : 0, workspace->data_ptr(), (size_t)workspace->numel(), 1, st),
+                     "fbev_backward_gather_stored");
+        else
+            raise_on(fbev_backward_gather_persistent(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(),
+                                                     image_feats.data_ptr(), projection_matrices.data_ptr<float>(), dd, df,
+                                                     accumulate ? 1 : 0, workspace->data_ptr(), (size_t)workspace->numel(), st),
+                     "fbev_backward_gather_persistent");
     } else if (backward_mode == 1) {
         raise_on(fbev_backward(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
                                projection_matrices.data_ptr<float>(), dd, df, accumulate ? 1 : 0, st),
@@ -486,7 +532,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("optimize_z_precompute"), py::arg("use_warp_kernel"), py::arg("use_vectorized_load"),
           py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f, py::arg("depth_min") = 1.0f,
           py::arg("depth_step") = 1.0f, py::arg("reduction") = 0, py::arg("count_out") = py::none(),
-          py::arg("geometry_cache") = py::none());
+          py::arg("geometry_cache") = py::none(), py::arg("sample_store") = py::none());
+    m.def("sample_store_bytes", &sample_store_bytes,
+          "bytes of the sample store a differentiated forward may fill for the backward (0: none for this problem)");
     m.def("build_geometry_cache", &build_geometry_cache,
           "per-cell lists of the samples in view, for flash_bevpool_forward(..., geometry_cache=...)",
           py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
@@ -498,7 +546,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("depth_distribution"), py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f,
           py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0,
           py::arg("backward_mode") = 0, py::arg("pair_capacity") = -1, py::arg("cell_count") = py::none(),
-          py::arg("accumulate") = true, py::arg("workspace") = py::none());
+          py::arg("accumulate") = true, py::arg("workspace") = py::none(), py::arg("sample_store") = py::none());
     m.def("backward_workspace_bytes", &backward_workspace_bytes,
           "bytes of a persistent inverse-map workspace (0 when the problem is beyond the inverse map)");
     m.def("prepare_backward_workspace", &prepare_backward_workspace,

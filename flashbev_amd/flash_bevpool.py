@@ -100,6 +100,22 @@ def _persistent_workspace(ext, depth_params, image_feats, projection_matrices, f
     return key, ws
 
 
+def _sample_store_limit() -> int:
+    """Largest sample store (bytes) a differentiated forward fills for its backward; FLASHBEV_SAMPLE_STORE_MB
+    (default 64, 0 switches it off).  The store holds a 32-byte record for every (cell, camera, height) sample slot
+    (25 MB on a 128 x 128 x 8 grid with six cameras) and lives, like a saved tensor, until the backward has run;
+    it pays where a call is bound by latency, i.e. on small grids."""
+    return int(float(os.environ.get("FLASHBEV_SAMPLE_STORE_MB", "64")) * 2 ** 20)
+
+
+@functools.lru_cache(maxsize=256)
+def _sample_store_bytes(cells_padded: int, samples_per_cell: int, texels: int) -> int:
+    """What fbev_sample_store_bytes answers: a slot of N * gz records per cell of the tiled walk."""
+    if texels >= 2 ** 29:
+        return 0
+    return cells_padded * samples_per_cell * 32
+
+
 # id(tensor) -> (weak reference, version, values, notes about the values).  Keyed by identity: a mapping keyed by the
 # tensors themselves would compare them with ``==`` on lookup, which is elementwise.
 _host_cache: dict = {}
@@ -235,16 +251,24 @@ class FlashBEVPool(torch.autograd.Function):
         wants_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         counts = torch.empty((B, grid[1], grid[0]), dtype=torch.float32,
                              device=image_feats.device) if wants_grad else None
+        # small problems also leave their kept samples behind, so that the backward's cell pass need not evaluate
+        # them again (the inverse-map backward only; not on cached geometry)
+        store = None
+        if wants_grad and geometry_cache is None and _backward_mode() in (0, 2):
+            nbytes = _sample_store_bytes(B * ((grid[0] + 7) // 8) * ((grid[1] + 7) // 8) * 64, N * grid[2], B * N * H * W)
+            if 0 < nbytes <= _sample_store_limit():
+                store = torch.empty(nbytes, dtype=torch.uint8, device=image_feats.device)
         ext.flash_bevpool_forward(
             depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
             vsize[0], vsize[1], vsize[2], vmin[0], vmin[1], vmin[2], out, out.numel(),
             depth_distribution, bool(use_shared_memory), bool(optimize_z_precompute),
             bool(use_warp_kernel), bool(use_vectorized_load), float(epsilon),
-            float(depth_weight_threshold), d_min, d_step, red, counts, geometry_cache)
+            float(depth_weight_threshold), d_min, d_step, red, counts, geometry_cache, store)
 
         if wants_grad:
             ctx.save_for_backward(depth_params, image_feats, projection_matrices)
             ctx.counts = counts
+            ctx.sample_store = store
             ctx.pair_capacity = _pair_capacity(B, N, grid)
             ctx.host = (fs_host, image_t, roi_t, grid_t)
             ctx.total_threads = out.numel()
@@ -280,7 +304,7 @@ class FlashBEVPool(torch.autograd.Function):
                     fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
                     ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
                     ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, ctx.pair_capacity, ctx.counts, False,
-                    ws)
+                    ws, ctx.sample_store if mode in (0, 2) else None)
             except Exception:
                 _workspaces.pop(key, None)       # a failed call leaves a persistent workspace undefined
                 raise

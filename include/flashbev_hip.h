@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FBEV_ABI_VERSION 8
+#define FBEV_ABI_VERSION 9
 
 typedef enum fbev_status {
     FBEV_OK = 0,
@@ -177,6 +177,31 @@ int fbev_backward_workspace_init(const fbev_problem *p, void *workspace, size_t 
 int fbev_backward_gather_persistent(const fbev_problem *p, const float *grad_out, const void *depth,
                                     const void *feats, const float *proj, float *d_depth, float *d_feats,
                                     int accumulate, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Forward and backward of one differentiated call sharing the sample evaluation.  fbev_forward_store is
+ * fbev_forward (same `out`, same `count_out`, which is required here) that also leaves, for every kept
+ * sample, a 32-byte record (bilinear fractions, first corner texel with the two clamp flags, depth weight
+ * and its two derivative terms, depth bins) in `store`: caller-owned device memory of
+ * fbev_sample_store_bytes(p) bytes, 16-byte aligned, one slot of N * grid_z records per BEV cell, i.e.
+ * B * ceil(gx/8) * ceil(gy/8) * 64 * N * grid_z * 32 bytes (0: outside the limits, B*N*H*W >= 2^29); only the
+ * records of kept samples are written.  fbev_backward_gather_stored is fbev_backward_gather (persistent == 0)
+ * or fbev_backward_gather_persistent (persistent != 0, `workspace` prepared as described there) whose cell
+ * pass copies those records instead of projecting and weighting every sample again; `cell_count` and `store`
+ * are what fbev_forward_store wrote for the same p, depth, feats and proj.  Same gradients as
+ * fbev_backward_gather, to rounding.  It pays where a call is bound by latency rather than throughput (small
+ * grids); the store is per-call state, like a tensor saved for the backward, and nothing checks that it
+ * belongs to these inputs: records that cannot have come from this problem are clamped, so a wrong buffer
+ * gives wrong numbers, never an access out of bounds.  No counterpart in the reference, whose backward
+ * recomputes every sample per channel thread (flashbev/flashbevpool/src/flash_bevpool_cuda.cu:448-568).
+ */
+size_t fbev_sample_store_bytes(const fbev_problem *p);
+int fbev_forward_store(const fbev_problem *p, const void *depth, const void *feats, const float *proj, float *out,
+                       float *count_out, void *store, size_t store_bytes, void *stream);
+int fbev_backward_gather_stored(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                                const float *proj, const float *cell_count, const void *store, size_t store_bytes,
+                                float *d_depth, float *d_feats, int accumulate, void *workspace, size_t workspace_bytes,
+                                int persistent, void *stream);
 
 /*
  * fbev_backward_gather without a workspace argument and without any allocation: the inverse map

@@ -108,11 +108,14 @@ def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEA
     per-texel segments; "gather_counted" defaults to half of that, the exactly packed layout), "columns" =
     fbev_backward_columns overwriting NaN-filled buffers with recounted cell counts, "persistent" =
     fbev_backward_gather_persistent on a workspace prepared once (three calls in a row, the last one returned),
-    "columns_acc" = the same accumulating into zero-filled buffers with the forward's counts."""
+    "columns_acc" = the same accumulating into zero-filled buffers with the forward's counts,
+    "stored" / "stored_persistent" = fbev_forward_store (whose output and counts must equal fbev_forward's bit
+    for bit) followed by fbev_backward_gather_stored on a per-call / a persistent workspace (twice in a row on
+    the persistent one)."""
     p = problem_for(x, w, dist, thr, eps, reduction)
     dev = x["image_feats"].device
     overwrite = mode in ("columns", "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite",
-                         "persistent_overwrite")
+                         "persistent_overwrite", "stored_overwrite", "stored_persistent_overwrite")
     fill = float("nan") if overwrite else 0.0
     dd = torch.full(x["depth_params"].shape, fill, dtype=torch.float32, device=dev) if want[0] else None
     df = torch.full(x["image_feats"].shape, fill, dtype=torch.float32, device=dev) if want[1] else None
@@ -135,6 +138,36 @@ def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEA
             _, cnt = capi_forward(x, w, dist, thr, eps, reduction, with_count=True)
             capi.check(capi.backward_columns(p, *args, cnt.data_ptr(), ddp, dfp, True, None, 0, st),
                        "fbev_backward_columns")
+    elif mode.startswith("stored"):
+        persistent = "persistent" in mode
+        out, cnt = capi_forward(x, w, dist, thr, eps, reduction, with_count=True)
+        sbytes = capi.sample_store_bytes(p)
+        assert sbytes > 0
+        store = torch.empty(sbytes, dtype=torch.uint8, device=dev).fill_(0xFF)      # unwritten records: texel far out of range
+        out2 = torch.full_like(out, float("nan"))
+        cnt2 = torch.full_like(cnt, float("nan"))
+        capi.check(capi.forward_store(p, x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
+                                      x["projection_matrices"].data_ptr(), out2.data_ptr(), cnt2.data_ptr(),
+                                      store.data_ptr(), sbytes, st), "fbev_forward_store")
+        torch.cuda.synchronize()
+        assert torch.equal(out2, out) and torch.equal(cnt2, cnt), "fbev_forward_store differs from fbev_forward"
+        if persistent:
+            nbytes = capi.backward_persistent_workspace_bytes(p)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(0x5A)
+            capi.check(capi.backward_workspace_init(p, ws.data_ptr(), nbytes, st), "fbev_backward_workspace_init")
+        else:
+            nbytes = capi.backward_workspace_bytes(p, capi.backward_max_pairs(p) if pair_capacity is None else pair_capacity)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        for call in range(2 if persistent else 1):
+            if dd is not None:
+                dd.fill_(fill)
+            if df is not None:
+                df.fill_(fill)
+            capi.check(capi.backward_gather_stored(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
+                                                   x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(),
+                                                   cnt2.data_ptr(), store.data_ptr(), sbytes, ddp, dfp, ws.data_ptr(), nbytes,
+                                                   st, accumulate=not overwrite, persistent=persistent),
+                       "fbev_backward_gather_stored")
     elif mode in ("persistent", "persistent_overwrite"):
         # a workspace prepared once, then three calls in a row on it (the claim-counter sets alternate);
         # the last call's gradients are returned

@@ -78,7 +78,9 @@ def test_forward_against_the_oracle_at_the_configurations_own_shape(name, gz, di
 BACKWARD_CASES = [("cfg4_hires", 1, "gather"), ("cfg4_hires", 2, "gather"), ("cfg5_train", 1, "gather"),
                   ("cfg5_train", 2, "gather"), ("cfg5_train", 0, "gather_counted"), ("cfg5_train", 1, "columns"),
                   ("cfg2_surround", 1, "persistent_overwrite"), ("cfg3_zsweep", 1, "persistent"),
-                  ("cfg4_hires", 2, "persistent_overwrite"), ("cfg5_train", 1, "persistent_overwrite")]
+                  ("cfg4_hires", 2, "persistent_overwrite"), ("cfg5_train", 1, "persistent_overwrite"),
+                  ("cfg3_zsweep", 2, "stored_persistent_overwrite"), ("cfg4_hires", 1, "stored"),
+                  ("cfg5_train", 0, "stored_persistent_overwrite")]
 
 
 @pytest.mark.parametrize("name,dist,mode", BACKWARD_CASES)

@@ -59,7 +59,8 @@ def test_forward_matches_c_oracle(name, dist, thr):
 @pytest.mark.parametrize("dist", [0, 1, 2])
 @pytest.mark.parametrize("mode", ["scatter", "gather", "gather_counted", "columns", "columns_acc",
                                   "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite",
-                                  "persistent", "persistent_overwrite"])
+                                  "persistent", "persistent_overwrite", "stored", "stored_overwrite",
+                                  "stored_persistent", "stored_persistent_overwrite"])
 def test_backward_matches_c_oracle(name, dist, mode):
     w, x = _inputs(name, dist)
     dd, df = U.capi_backward(x, w, dist, mode=mode)
@@ -79,11 +80,52 @@ def test_backward_gather_with_short_workspace(capacity):
     assert U.violations(dd.cpu().numpy(), want_dd)[0] == 0
 
 
+@pytest.mark.parametrize("capacity", [0, 1000, 100000])
+def test_backward_from_the_sample_store_with_short_workspace(capacity):
+    """The same through the samples the forward stored: whatever finds no room in the counted layout is added
+    with atomics by the cell pass."""
+    w, x = _inputs("cfg2_surround", 2)
+    dd, df = U.capi_backward(x, w, 2, mode="stored", pair_capacity=capacity)
+    want_dd, want_df = U.oracle_backward(x, w, 2)
+    assert U.violations(df.cpu().numpy(), want_df)[0] == 0
+    assert U.violations(dd.cpu().numpy(), want_dd)[0] == 0
+
+
+def test_a_foreign_sample_store_gives_no_access_out_of_bounds():
+    """Records that cannot have come from a forward of this problem (counts beyond N * gz, texels beyond the
+    feature maps) are clamped and zeroed by the cell pass: wrong numbers, but a normal return and finite
+    gradients.  (Nothing ties a store to its inputs; this only pins that the guard holds.)"""
+    w, x = _inputs("cfg1_tiny", 1)
+    p = U.problem_for(x, w, 1)
+    dev = x["image_feats"].device
+    st = torch.cuda.current_stream().cuda_stream
+    sbytes = capi.sample_store_bytes(p)
+    store = torch.full((sbytes,), 0x7F, dtype=torch.uint8, device=dev)            # texel index 0x1fdfdfdf, far out of range
+    cnt = torch.full((p.batch, p.grid_y, p.grid_x), 1.0e9, dtype=torch.float32, device=dev)
+    dd = torch.full(x["depth_params"].shape, float("nan"), dtype=torch.float32, device=dev)
+    df = torch.full(x["image_feats"].shape, float("nan"), dtype=torch.float32, device=dev)
+    nbytes = capi.backward_workspace_bytes(p, capi.backward_max_pairs(p))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    capi.check(capi.backward_gather_stored(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
+                                           x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(), cnt.data_ptr(),
+                                           store.data_ptr(), sbytes, dd.data_ptr(), df.data_ptr(), ws.data_ptr(), nbytes, st,
+                                           accumulate=False), "fbev_backward_gather_stored")
+    torch.cuda.synchronize()
+    assert torch.isfinite(dd).all() and torch.isfinite(df).all()
+    # and the argument checks: a short store, a missing count
+    assert capi.backward_gather_stored(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
+                                       x["projection_matrices"].data_ptr(), cnt.data_ptr(), store.data_ptr(), sbytes - 32,
+                                       dd.data_ptr(), df.data_ptr(), ws.data_ptr(), nbytes, st) == -2
+    assert capi.backward_gather_stored(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
+                                       x["projection_matrices"].data_ptr(), None, store.data_ptr(), sbytes, dd.data_ptr(),
+                                       df.data_ptr(), ws.data_ptr(), nbytes, st) == -1
+
+
 def test_backward_single_gradient():
     """Either gradient pointer may be NULL."""
     w, x = _inputs("cfg2_surround", 0)
     want_dd, want_df = U.oracle_backward(x, w, 0)
-    for mode in ("scatter", "gather", "gather_counted", "columns"):
+    for mode in ("scatter", "gather", "gather_counted", "columns", "stored", "stored_persistent"):
         dd, df = U.capi_backward(x, w, 0, mode=mode, want=(True, False))
         assert df is None and U.violations(dd.cpu().numpy(), want_dd)[0] == 0
         dd, df = U.capi_backward(x, w, 0, mode=mode, want=(False, True))

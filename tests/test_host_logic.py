@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in flashbev_hip.h but not exported"
     assert sorted(capi.EXPORTS) == names
-    assert lib.fbev_abi_version() == 8
+    assert lib.fbev_abi_version() == 9
     assert lib.fbev_problem_size() == ctypes.sizeof(capi.FbevProblem)
 
 
@@ -189,6 +189,33 @@ def fake_ext(monkeypatch):
     return ext
 
 
+def test_sample_store_goes_with_small_differentiated_calls_only(fake_ext, monkeypatch):
+    """A differentiated forward of a small problem hands the extension a sample store and the backward gets the same
+    tensor; an inference call, a problem beyond FLASHBEV_SAMPLE_STORE_MB and the column-owner backward get none."""
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    args = (x["depth_params"], x["projection_matrices"], x["feature_size"], x["image_size"], x["roi_range"], x["grid_size"])
+
+    def call(grad):
+        f = x["image_feats"].clone().requires_grad_(grad)
+        out = flash_bevpool(f, *args)
+        if grad:
+            out.sum().backward()
+        return fake_ext.fwd[-1]
+
+    store = call(True)
+    gx, gy, gz = w.grid_size
+    want = w.batch * ((gx + 7) // 8) * ((gy + 7) // 8) * 64 * w.num_cams * gz * 32
+    assert store is not None and store.dtype == torch.uint8 and store.numel() == want
+    assert fake_ext.bwd[-1] is store
+    assert call(False) is None
+    monkeypatch.setenv("FLASHBEV_SAMPLE_STORE_MB", str((want - 1) / 2 ** 20))
+    assert call(True) is None and fake_ext.bwd[-1] is None
+    monkeypatch.setenv("FLASHBEV_SAMPLE_STORE_MB", "64")
+    monkeypatch.setenv("FLASHBEV_BACKWARD", "columns")
+    assert call(True) is None and fake_ext.bwd[-1] is None
+
+
 def test_operator_marshalling_matches_reference_order(fake_ext):
     w = WORKLOADS["cfg1_tiny"]
     x = make_inputs(w, "parametric")
@@ -220,7 +247,7 @@ def test_persistent_workspace_is_prepared_once_per_shape_and_dropped_when_switch
         out = flash_bevpool(f, x["depth_params"], x["projection_matrices"], x["feature_size"], x["image_size"],
                             x["roi_range"], x["grid_size"] if grid is None else grid)
         out.sum().backward()
-        return fake_ext.bwd[-1]
+        return fake_ext.bwd[-2]
 
     ws = step()
     assert ws is not None and ws.dtype == torch.uint8 and fake_ext.prepared == 1
@@ -259,13 +286,13 @@ def test_forward_without_gradients_skips_the_autograd_function(fake_ext, monkeyp
     real_apply = FlashBEVPool.apply
     monkeypatch.setattr(FlashBEVPool, "apply", lambda *a: applied.append(1) or real_apply(*a))
     out = flash_bevpool(x["image_feats"], *base)
-    assert not applied and not out.requires_grad and fake_ext.fwd[-2] is None        # no count buffer
+    assert not applied and not out.requires_grad and fake_ext.fwd[-3] is None        # no count buffer
     f = x["image_feats"].clone().requires_grad_(True)
     with torch.no_grad():
         out = flash_bevpool(f, *base)
     assert not applied and not out.requires_grad
     out = flash_bevpool(f, *base)
-    assert applied and out.requires_grad and fake_ext.fwd[-2] is not None
+    assert applied and out.requires_grad and fake_ext.fwd[-3] is not None
 
 
 def test_half_inputs_are_not_upcast_and_mixed_dtypes_are(fake_ext):
