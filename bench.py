@@ -130,7 +130,7 @@ class Runner:
             x["grad_out"], x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
             x["image_size"], x["roi_range"], x["grid_size"], self.d_depth, self.d_feats, self.out.numel(),
             self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0, self.backward_mode, -1,
-            self.counts, False, self.workspace, self.store if self.stored_by_forward else None)
+            self.counts, False, self.workspace, self.store if self.stored_by_forward else None, list(self.vsize))
 
 
 # Untimed steps of the workload itself, run for this many milliseconds before the warm-up steps of every

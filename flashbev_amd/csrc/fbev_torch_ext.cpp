@@ -262,15 +262,22 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                             int64_t total_threads, int depth_distribution, float epsilon, float depth_weight_threshold,
                             float depth_min, float depth_step, int reduction, int backward_mode,
                             int64_t pair_capacity, std::optional<at::Tensor> cell_count, bool accumulate,
-                            std::optional<at::Tensor> workspace, std::optional<at::Tensor> sample_store) {
+                            std::optional<at::Tensor> workspace, std::optional<at::Tensor> sample_store,
+                            std::optional<std::vector<double>> voxel_size) {
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
     auto roi = host_floats(roi_range, 6, "roi_range");
     const int32_t g[3] = {p.grid_x, p.grid_y, p.grid_z};
+    TORCH_CHECK(!voxel_size.has_value() || voxel_size->size() == 3, "flashbevpool_ext: voxel_size needs 3 entries");
     for (int a = 0; a < 3; ++a) {
-        // float64 arithmetic on the fp32 bounds, exactly what the Python operator hands the forward
         p.voxel_min[a] = (double)roi[2 * a];
-        p.voxel_size[a] = ((double)roi[2 * a + 1] - (double)roi[2 * a]) / (double)g[a];
+        // The cell size must be the one the forward was given, or forward and backward would disagree on
+        // samples that sit within rounding of a border.  A caller that names it (the Python operator passes the
+        // float64 quotient of the fp32 bounds to both) is taken at its word.  The reference's 14 positional
+        // arguments carry no size: its Python forms fp32((max - min) / grid) on the fp32 tensor and hands that
+        // to the forward (flash_bevpool.py:62-64), so that is what an unnamed size means here.
+        p.voxel_size[a] = voxel_size.has_value() ? (*voxel_size)[a]
+                                                 : (double)((float)(roi[2 * a + 1] - roi[2 * a]) / (float)g[a]);
     }
     check_dev(out_grad, depth_params, "out_grad");
     TORCH_CHECK(out_grad.scalar_type() == at::kFloat, "flashbevpool_ext: out_grad must be float32");
@@ -546,7 +553,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("depth_distribution"), py::arg("epsilon") = 1e-6f, py::arg("depth_weight_threshold") = 1e-6f,
           py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0,
           py::arg("backward_mode") = 0, py::arg("pair_capacity") = -1, py::arg("cell_count") = py::none(),
-          py::arg("accumulate") = true, py::arg("workspace") = py::none(), py::arg("sample_store") = py::none());
+          py::arg("accumulate") = true, py::arg("workspace") = py::none(), py::arg("sample_store") = py::none(),
+          py::arg("voxel_size") = py::none());
     m.def("backward_workspace_bytes", &backward_workspace_bytes,
           "bytes of a persistent inverse-map workspace (0 when the problem is beyond the inverse map)");
     m.def("prepare_backward_workspace", &prepare_backward_workspace,

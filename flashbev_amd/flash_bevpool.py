@@ -269,6 +269,7 @@ class FlashBEVPool(torch.autograd.Function):
             ctx.save_for_backward(depth_params, image_feats, projection_matrices)
             ctx.counts = counts
             ctx.sample_store = store
+            ctx.voxel_size = list(vsize)          # the backward takes the cell size the forward was given
             ctx.pair_capacity = _pair_capacity(B, N, grid)
             ctx.host = (fs_host, image_t, roi_t, grid_t)
             ctx.total_threads = out.numel()
@@ -304,7 +305,7 @@ class FlashBEVPool(torch.autograd.Function):
                     fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
                     ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
                     ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, ctx.pair_capacity, ctx.counts, False,
-                    ws, ctx.sample_store if mode in (0, 2) else None)
+                    ws, ctx.sample_store if mode in (0, 2) else None, ctx.voxel_size)
             except Exception:
                 _workspaces.pop(key, None)       # a failed call leaves a persistent workspace undefined
                 raise

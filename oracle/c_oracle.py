@@ -33,6 +33,7 @@ class OracleProblem(ctypes.Structure):
         ("dist", ctypes.c_int32), ("D", ctypes.c_int32),
         ("dmin", ctypes.c_float), ("dstep", ctypes.c_float),
         ("reduce_sum", ctypes.c_int32),
+        ("step", ctypes.c_double * 3),
     ]
 
 
@@ -83,7 +84,7 @@ def _proj34(proj) -> np.ndarray:
 def make_problem(depth_shape, feat_shape, image_size: Sequence[int], roi_range: Sequence[float],
                  grid_size: Sequence[int], depth_distribution: int, epsilon: float,
                  depth_weight_threshold: float, depth_range=(1.0, 1.0),
-                 reduce_sum: bool = False) -> OracleProblem:
+                 reduce_sum: bool = False, voxel_size=None) -> OracleProblem:
     B, N, H, W, C = feat_shape
     assert tuple(depth_shape[:4]) == (B, N, H, W)
     p = OracleProblem()
@@ -100,6 +101,9 @@ def make_problem(depth_shape, feat_shape, image_size: Sequence[int], roi_range: 
         assert p.D == 2
     p.dmin, p.dstep = float(depth_range[0]), float(depth_range[1])
     p.reduce_sum = int(bool(reduce_sum))
+    # the cell size a caller insists on (None: the float64 quotient of the bounds, the canonical one)
+    for i in range(3):
+        p.step[i] = 0.0 if voxel_size is None else float(voxel_size[i])
     return p
 
 
@@ -126,11 +130,11 @@ def geometry(proj, feat_hw, image_size, roi_range, grid_size, epsilon=1e-6):
 
 def forward(depth, feats, proj, image_size, roi_range, grid_size, depth_distribution=0,
             epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=(1.0, 1.0), reduce_sum=False,
-            return_aux=False):
+            return_aux=False, voxel_size=None):
     """out [B,gy,gx,C] float32 (and optionally per-cell counts and the kept-sample mask)."""
     depth, feats, P = _f32(depth), _f32(feats), _proj34(proj)
     prob = make_problem(depth.shape, feats.shape, image_size, roi_range, grid_size,
-                        depth_distribution, epsilon, depth_weight_threshold, depth_range, reduce_sum)
+                        depth_distribution, epsilon, depth_weight_threshold, depth_range, reduce_sum, voxel_size)
     out = np.zeros((prob.B, prob.gy, prob.gx, prob.C), np.float32)
     cnt = np.zeros((prob.B, prob.gy, prob.gx), np.float32)
     keep = np.zeros((prob.B, prob.gy, prob.gx, prob.N, prob.gz), np.uint8)
@@ -142,11 +146,11 @@ def forward(depth, feats, proj, image_size, roi_range, grid_size, depth_distribu
 
 
 def backward(grad_out, depth, feats, proj, image_size, roi_range, grid_size, depth_distribution=0,
-             epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=(1.0, 1.0), reduce_sum=False):
+             epsilon=1e-6, depth_weight_threshold=1e-6, depth_range=(1.0, 1.0), reduce_sum=False, voxel_size=None):
     """(d_depth, d_feats): exact gradient of ``forward``, float64 sums rounded to float32."""
     depth, feats, P, go = _f32(depth), _f32(feats), _proj34(proj), _f32(grad_out)
     prob = make_problem(depth.shape, feats.shape, image_size, roi_range, grid_size,
-                        depth_distribution, epsilon, depth_weight_threshold, depth_range, reduce_sum)
+                        depth_distribution, epsilon, depth_weight_threshold, depth_range, reduce_sum, voxel_size)
     assert go.shape == (prob.B, prob.gy, prob.gx, prob.C)
     d_depth = np.zeros_like(depth)
     d_feats = np.zeros_like(feats)

@@ -25,11 +25,13 @@
  * parity unpinned by the reference; it is pinned only by the dense restatement and
  * the invariants in tests/.
  *
- * Pinning of this file (see tests/test_oracle_*.py): brute-force float64 Python loops
- * on tiny grids, torch grid_sample(bilinear, border, align_corners=True) as the
- * library routine the interpolation reduces to, closed forms (optical-axis point,
- * integer sample positions, likelihood at the mean), linearity / adjoint identities,
- * and float64 finite differences for the gradients.
+ * Pinning of this file (tests/test_oracle_pinning.py): closed-form projections in
+ * binary-friendly numbers (optical-axis point, behind the camera, the last-column clamp),
+ * textbook likelihood values at the mean and at one sigma, threshold and categorical-bin
+ * cases, torch grid_sample(bilinear, border, align_corners=True) as the library routine
+ * the interpolation reduces to (this file against the dense path, up to the benchmark's
+ * largest shapes), linearity / constant-feature / camera-permutation invariants, and for
+ * the gradients float64 autograd, gradcheck, central differences and the adjoint identity.
  */
 #include <math.h>
 #include <stdint.h>
@@ -48,6 +50,7 @@ typedef struct {
     int32_t D;         /* channels of the depth tensor: 2, or number of bins */
     float dmin, dstep; /* categorical: bin k sits at dmin + k*dstep */
     int32_t reduce_sum;/* 0: mean over valid samples (reference), 1: plain sum */
+    double step[3];    /* cell size along x, y, z; 0: (hi - lo) / n in float64 (the canonical one) */
 } oracle_problem;
 
 typedef struct {
@@ -100,9 +103,11 @@ static inline void project_sample(const oracle_problem *p, const float *P,
  * of the fp32 step along the axis (0.8 m is not an fp32 number), which a Gaussian tail weight
  * magnifies beyond the parity tolerance, so the correctly rounded centre is the canonical one.
  */
-static inline float voxel_centre(float lo, float hi, int n, int i)
+static inline float voxel_centre(float lo, float hi, int n, int i, double given_step)
 {
-    double step = ((double)hi - (double)lo) / (double)n;
+    /* (a caller of the operator's extension may hand over its own cell size, e.g. the fp32 quotient the
+     * reference's Python forms, flash_bevpool.py:62-64: then that size is the step) */
+    double step = given_step > 0.0 ? given_step : ((double)hi - (double)lo) / (double)n;
     return (float)((double)lo + ((double)i + 0.5) * step);
 }
 
@@ -170,11 +175,11 @@ void fbev_oracle_geometry(const oracle_problem *p, const float *proj /* [B,N,12]
     for (int b = 0; b < p->B; ++b)
         for (int iy = 0; iy < p->gy; ++iy)
             for (int ix = 0; ix < p->gx; ++ix) {
-                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix);
-                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy);
+                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix, p->step[0]);
+                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy, p->step[1]);
                 for (int n = 0; n < p->N; ++n)
                     for (int iz = 0; iz < p->gz; ++iz, ++s) {
-                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz);
+                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz, p->step[2]);
                         sample_geom g;
                         project_sample(p, proj + ((size_t)b * p->N + n) * 12, x, y, z, &g);
                         if (mask) mask[s] = (uint8_t)g.valid;
@@ -207,8 +212,8 @@ void fbev_oracle_forward(const oracle_problem *p, const float *depth, const floa
     for (int b = 0; b < p->B; ++b)
         for (int iy = 0; iy < p->gy; ++iy)
             for (int ix = 0; ix < p->gx; ++ix) {
-                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix);
-                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy);
+                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix, p->step[0]);
+                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy, p->step[1]);
                 for (int c = 0; c < C; ++c) acc[c] = 0.0f;
                 float cnt = 0.0f;
                 for (int n = 0; n < p->N; ++n) {
@@ -216,7 +221,7 @@ void fbev_oracle_forward(const oracle_problem *p, const float *depth, const floa
                     const float *dcam = depth + cam * H * W * p->D;
                     const float *fcam = feats + cam * H * W * C;
                     for (int iz = 0; iz < p->gz; ++iz, ++s) {
-                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz);
+                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz, p->step[2]);
                         sample_geom g;
                         if (keep) keep[s] = 0;
                         project_sample(p, proj + cam * 12, x, y, z, &g);
@@ -262,14 +267,14 @@ void fbev_oracle_backward(const oracle_problem *p, const float *grad_out, const 
     for (int b = 0; b < p->B; ++b)
         for (int iy = 0; iy < p->gy; ++iy)
             for (int ix = 0; ix < p->gx; ++ix) {
-                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix);
-                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy);
+                float x = voxel_centre(p->roi[0], p->roi[1], p->gx, ix, p->step[0]);
+                float y = voxel_centre(p->roi[2], p->roi[3], p->gy, iy, p->step[1]);
                 int cnt = 0;
                 for (int n = 0; n < p->N; ++n) {
                     size_t cam = (size_t)b * p->N + n;
                     for (int iz = 0; iz < p->gz; ++iz) {
                         int k = n * p->gz + iz;
-                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz);
+                        float z = voxel_centre(p->roi[4], p->roi[5], p->gz, iz, p->step[2]);
                         project_sample(p, proj + cam * 12, x, y, z, &gs[k]);
                         es[k].keep = 0;
                         if (!gs[k].valid) continue;

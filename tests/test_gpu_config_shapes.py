@@ -129,6 +129,50 @@ def test_forward_on_cached_geometry_equals_the_forward_bit_for_bit_and_the_oracl
         assert int(counts.sum().item()) == int(geo["mask"].sum())
 
 
+PHASE_A_CASES = [("cfg1_tiny", None, 0), ("cfg2_surround", None, 0), ("cfg3_zsweep", 12, 0), ("cfg4_hires", None, 2),
+                 ("cfg5_train", None, 5)]
+
+
+@pytest.mark.parametrize("name,gz,b", PHASE_A_CASES)
+def test_the_sample_phases_own_indices_and_fractions_equal_the_oracles_bit_for_bit(name, gz, b):
+    """The geometry cache is a dump of what the kernels' three-stage sample phase computes for every sample in
+    view (flash_bevpool_cuda.cu:137-159 in the reference): the bilinear fractions, the first corner texel with the
+    two clamp flags, and the depth along the optical axis, per cell in (camera, height) order.  Decoded and compared
+    with the oracle's per-sample geometry as bits: the same samples in view, the same indices, the same fractions and
+    depths, at every cell of one batch element."""
+    w = workload(name, gz)
+    x = make_inputs(w, "parametric", device="cuda")
+    cache = U.capi_geometry_cache(x, w, 1)
+    head = cache[:48].view(torch.int32).cpu().tolist()
+    padded, nz = head[8], head[9]
+    N, (H, W), (gx, gy, _) = w.num_cams, w.feat_hw, w.grid_size
+    assert nz == N * w.grid_size[2]
+    counts = cache[256 + 4 * b * padded:256 + 4 * (b + 1) * padded].view(torch.int32).cpu().numpy()
+    first = 256 + (4 * w.batch * padded + 255) // 256 * 256
+    rec = cache[first + 16 * b * padded * nz:first + 16 * (b + 1) * padded * nz].view(torch.int32).cpu().numpy().reshape(padded, nz, 4)
+    ref = c_oracle.geometry(x["projection_matrices"][b:b + 1].cpu().numpy(), w.feat_hw, w.image_hw, w.roi_range, w.grid_size)
+    mask = ref["mask"][0].reshape(gy * gx, nz).astype(bool)
+    # where a cell sits in the tiled walk (8 x 8 tiles, row-major inside and across tiles)
+    iy, ix = np.divmod(np.arange(gy * gx), gx)
+    q = ((iy // 8) * ((gx + 7) // 8) + ix // 8) * 64 + (iy % 8) * 8 + ix % 8
+    want_counts = np.zeros(padded, np.int32)
+    want_counts[q] = mask.sum(1)
+    assert mask.sum() > 0 and np.array_equal(counts, want_counts)
+    order = np.argsort(q)
+    sel = mask[order]                                                  # [cells in walk order, samples]
+    got = rec[q[order]][np.arange(nz)[None, :] < counts[q[order]][:, None]]      # the cells' lists, one after the other
+    idx = ref["idx"][0].reshape(gy * gx, nz, 4)[order][sel]            # (u0, u1, v0, v1)
+    frac = ref["frac"][0].reshape(gy * gx, nz, 2)[order][sel].view(np.int32)
+    depth = ref["depth"][0].reshape(gy * gx, nz)[order][sel].view(np.int32)
+    cam = np.broadcast_to(np.repeat(np.arange(N), w.grid_size[2])[None, :], (gy * gx, nz))[sel]
+    texel = ((b * N + cam) * H + idx[:, 2]) * W + idx[:, 0]
+    flags = (idx[:, 1] != idx[:, 0]).astype(np.int32) | ((idx[:, 3] != idx[:, 2]).astype(np.int32) << 1)
+    assert got.shape[0] == idx.shape[0]
+    assert np.array_equal(got[:, 0], frac[:, 0]) and np.array_equal(got[:, 1], frac[:, 1])
+    assert np.array_equal(got[:, 2], (texel << 2) | flags)
+    assert np.array_equal(got[:, 3], depth)
+
+
 def test_cached_geometry_rejects_short_caches_and_follows_new_matrices():
     w = workload("cfg2_surround")
     x = make_inputs(w, "parametric", device="cuda")

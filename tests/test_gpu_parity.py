@@ -221,6 +221,60 @@ def test_autograd_operator_matches_capi():
     assert U.violations(d.grad.cpu().numpy(), want_dd)[0] == 0
 
 
+@pytest.mark.parametrize("dist", [0, 1])
+def test_extension_called_the_way_the_references_python_calls_it(dist):
+    """flashbevpool_ext.flash_bevpool_forward / flash_bevpool_backward with exactly what the reference's operator
+    hands its extension (flashbev/flashbevpool/flash_bevpool.py:47-136): 21 and 14 positional arguments, device
+    tensors for feature_size, image_size, grid_size and roi_range, the three cell sizes as 0-dim fp32 tensors
+    fp32((max - min) / grid), caller-zeroed output and gradient buffers.  On the 200 x 200 grid 0.512 m is no fp32
+    number, so the fp32 size the forward receives differs from the float64 quotient; the backward, which receives
+    no size, must select the very samples the forward selected: both against the oracle run on that same fp32 size,
+    and the forward's cell counts against a recount the backward path makes from the region of interest."""
+    from flashbev_amd._native import load_ext
+    ext = load_ext()
+    w = WORKLOADS["cfg3_zsweep"].with_z(8)
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    depth_params = x["depth_params"].contiguous().float()
+    image_feats = x["image_feats"].contiguous().float()
+    projection_matrices = x["projection_matrices"].contiguous().float()
+    dev = image_feats.device
+    feature_size = torch.tensor(w.feat_hw, dtype=torch.int32, device=dev).repeat(w.batch, w.num_cams, 1).contiguous().int()
+    image_size = torch.tensor(w.image_hw, device=dev).contiguous().int()
+    roi_range = torch.tensor(w.roi_range, device=dev).contiguous().float()
+    grid_size = torch.tensor(w.grid_size, device=dev).contiguous().int()
+    grid_x, grid_y, grid_z = grid_size[0].item(), grid_size[1].item(), grid_size[2].item()
+    voxel_size_x = (roi_range[1] - roi_range[0]) / grid_x
+    voxel_size_y = (roi_range[3] - roi_range[2]) / grid_y
+    voxel_size_z = (roi_range[5] - roi_range[4]) / grid_z
+    assert voxel_size_x.dim() == 0 and voxel_size_x.dtype == torch.float32
+    r32 = np.float32(w.roi_range)
+    assert float(voxel_size_x) != (float(r32[1]) - float(r32[0])) / w.grid_size[0]      # the case this test is about
+    out = image_feats.new_zeros((w.batch, grid_size[1], grid_size[0], w.channels))
+    ext.flash_bevpool_forward(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              voxel_size_x, voxel_size_y, voxel_size_z, roi_range[0].item(), roi_range[2].item(),
+                              roi_range[4].item(), out, out.numel(), dist, True, True, False, False, 1e-6, 1e-6)
+    depth_params_grad = torch.zeros_like(depth_params)
+    image_feats_grad = torch.zeros_like(image_feats)
+    ext.flash_bevpool_backward(x["grad_out"], depth_params, image_feats, projection_matrices, feature_size, image_size,
+                               roi_range, grid_size, depth_params_grad, image_feats_grad, out.numel(), dist, 1e-6, 1e-6)
+    torch.cuda.synchronize()
+    sizes = [float(voxel_size_x), float(voxel_size_y), float(voxel_size_z)]
+    want, cnt, _ = U.oracle_forward(x, w, dist, return_aux=True, voxel_size=sizes)
+    bad, maxabs, ratio = U.violations(out.cpu().numpy(), want)
+    assert bad == 0, (bad, maxabs, ratio)
+    want_dd, want_df = U.oracle_backward(x, w, dist, voxel_size=sizes)
+    for got, ref, what in ((image_feats_grad, want_df, "d_feats"), (depth_params_grad, want_dd, "d_depth")):
+        bad, maxabs, ratio = U.violations(got.cpu().numpy(), ref)
+        assert bad == 0, (what, bad, maxabs, ratio)
+    # the same selection on both sides: the forward's counts (fp32 sizes) equal the oracle's for those sizes
+    counts = torch.empty((w.batch, w.grid_size[1], w.grid_size[0]), dtype=torch.float32, device=dev)
+    ext.flash_bevpool_forward(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              voxel_size_x, voxel_size_y, voxel_size_z, roi_range[0].item(), roi_range[2].item(),
+                              roi_range[4].item(), out, out.numel(), dist, True, True, False, False, 1e-6, 1e-6, 1.0, 1.0, 0,
+                              counts)
+    assert np.array_equal(counts.cpu().numpy(), cnt)
+
+
 @pytest.mark.parametrize("name,dist", [("gaussian", 0), ("laplace", 1), ("categorical", 2)])
 def test_kernels_against_the_committed_vectors(name, dist):
     """The tiny configuration against tests/golden/ (the oracle's outputs, committed): masks,

@@ -207,13 +207,13 @@ def test_sample_store_goes_with_small_differentiated_calls_only(fake_ext, monkey
     gx, gy, gz = w.grid_size
     want = w.batch * ((gx + 7) // 8) * ((gy + 7) // 8) * 64 * w.num_cams * gz * 32
     assert store is not None and store.dtype == torch.uint8 and store.numel() == want
-    assert fake_ext.bwd[-1] is store
+    assert fake_ext.bwd[-2] is store
     assert call(False) is None
     monkeypatch.setenv("FLASHBEV_SAMPLE_STORE_MB", str((want - 1) / 2 ** 20))
-    assert call(True) is None and fake_ext.bwd[-1] is None
+    assert call(True) is None and fake_ext.bwd[-2] is None
     monkeypatch.setenv("FLASHBEV_SAMPLE_STORE_MB", "64")
     monkeypatch.setenv("FLASHBEV_BACKWARD", "columns")
-    assert call(True) is None and fake_ext.bwd[-1] is None
+    assert call(True) is None and fake_ext.bwd[-2] is None
 
 
 def test_operator_marshalling_matches_reference_order(fake_ext):
@@ -247,7 +247,7 @@ def test_persistent_workspace_is_prepared_once_per_shape_and_dropped_when_switch
         out = flash_bevpool(f, x["depth_params"], x["projection_matrices"], x["feature_size"], x["image_size"],
                             x["roi_range"], x["grid_size"] if grid is None else grid)
         out.sum().backward()
-        return fake_ext.bwd[-2]
+        return fake_ext.bwd[-3]
 
     ws = step()
     assert ws is not None and ws.dtype == torch.uint8 and fake_ext.prepared == 1

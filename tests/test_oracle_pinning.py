@@ -203,6 +203,45 @@ def test_c_oracle_agrees_with_grid_sample_path(name, dist):
     assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["cosine"] > 0.9999, m
 
 
+# (configuration, height bins, depth model, bound on max |canonical fp32 - dense float64| over the output)
+LARGE_SHAPES = [("cfg3_zsweep", 16, 1, 5e-5), ("cfg4_hires", None, 1, 3e-4), ("cfg5_train", None, 1, 5e-5)]
+
+
+@pytest.mark.parametrize("name,gz,dist,max_abs", LARGE_SHAPES)
+def test_c_oracle_agrees_with_the_dense_path_at_the_large_shapes(name, gz, dist, max_abs):
+    """The named parity target at the benchmark's own sizes, as the reference's difference harness compares its
+    two paths there (tools/profile_differences.py:183-280): the height-bin sweep at 16 bins, and one batch element of
+    the bf16 and the fp16 configuration, whose inputs widen exactly, so that the dense path runs in fp32 and in
+    float64 on the very same values.  Masks and counts against the dense float64 evaluation; the output against the
+    dense fp32 path at rtol 1e-4 / atol 1e-5 with the dense path's own distance to float64 as the allowance (a
+    difference between two fp32 formulations cannot be held to less than one of them keeps against exact
+    arithmetic), the reference's mean-square, mean-absolute and cosine acceptance statistics, and the stated bound on max |difference| to float64."""
+    import dataclasses
+    w = WORKLOADS[name] if gz is None else WORKLOADS[name].with_z(gz)
+    x = make_inputs(w, "categorical" if dist == 2 else "parametric")
+    x = {k: (v[:1].contiguous() if torch.is_tensor(v) and v.dim() >= 4 else v) for k, v in x.items()}
+    w = dataclasses.replace(w, batch=1)
+    kw = U.op_kwargs(w, dist)
+    out_c, cnt_c, keep = U.oracle_forward(x, w, dist, return_aux=True)
+    dense = {}
+    for tag, cast in (("f32", lambda t: t.float()), ("f64", lambda t: t.double())):
+        out, cnt, fov = dense_torch.dense_pool(cast(x["image_feats"]), cast(x["depth_params"]),
+                                               cast(x["projection_matrices"]), return_aux=True, **kw)
+        dense[tag] = (out.numpy(), cnt.numpy(), fov.numpy())
+    g = c_oracle.geometry(x["projection_matrices"].numpy(), w.feat_hw, w.image_hw, w.roi_range, w.grid_size)
+    assert keep.sum() > 100000
+    assert (g["mask"] != dense["f64"][2]).sum() <= 2
+    assert (cnt_c != dense["f64"][1]).sum() <= 2
+    same = (cnt_c == dense["f64"][1]) & (cnt_c == dense["f32"][1])
+    ours = U.violations(out_c[same], dense["f32"][0][same])
+    floor = U.violations(dense["f32"][0][same], dense["f64"][0][same])
+    assert ours[0] <= floor[0] + 8 and ours[2] <= max(1.0, 1.5 * floor[2]), (ours, floor)
+    exact = U.violations(out_c[same], dense["f64"][0][same])
+    assert exact[1] <= max_abs, exact
+    m = U.reference_metrics(out_c, dense["f32"][0])
+    assert m["mse"] < 1e-6 and m["mae"] < 1e-6 and m["cosine"] > 0.9999, m
+
+
 def test_reduction_invariants():
     w = WORKLOADS["cfg2_surround"]
     x = make_inputs(w, "parametric")
