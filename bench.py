@@ -21,9 +21,10 @@ parameters, tools/config/config.yaml:29).  The single JSON line printed on stdou
                         events the library records around every one of its launches over a
                         second run of the same K steps, against the 8 TB/s HBM3E peak;
                         "kernels" lists every kernel's mean duration and launch count
-  other_workloads       the high-resolution inference and the training-size configurations timed in the
-                        same run (forward; forward and backward), with their compulsory bytes and
-                        fraction of the HBM peak: the sizes at which that fraction means something
+  other_workloads       the height-bin sweep (forward, 4 / 8 / 12 / 16 bins), the high-resolution inference and
+                        the training-size configurations timed in the same run (forward; forward and
+                        backward), with their compulsory bytes and fraction of the HBM peak (which means
+                        something at the two large sizes only)
   cpu_baseline          the dense PyTorch restatement of the reference's pooling path
                         (oracle/dense_torch.py), forward+backward via autograd on the host
                         cores, same workload -- a reported baseline, not a target.
@@ -57,11 +58,17 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 
 def measured_traffic(workload: str, depth: str, backward_mode: int):
+    """The counter-measured bytes of one workload, with the commit of the sources and the kernels they were
+    collected on (recorded in the file when it is written), so that a figure older than the kernels shows."""
     try:
         with open(TRAFFIC_FILE) as fh:
-            return json.load(fh).get(f"{workload}/{depth}/{backward_mode}")
+            table = json.load(fh)
     except (OSError, ValueError):
         return None
+    rec = table.get(f"{workload}/{depth}/{backward_mode}")
+    if rec is not None:
+        rec = dict(rec, commit=rec.get("commit", table.get("commit")))
+    return rec
 
 
 DIST_OF = {"gaussian": (0, "parametric"), "laplace": (1, "parametric"), "categorical": (2, "categorical")}
@@ -338,12 +345,14 @@ def cpu_baseline(w, depth_name: str, budget_s: float = 20.0, max_runs: int = 5):
 
 
 def other_workloads(steps: int, warmup: int, backward_mode: int):
-    """The two large configurations in the same run: high-resolution inference (bf16, forward) and
-    training size (fp16, forward and backward), Laplace depth; event-timed calls, compulsory bytes
-    (every operand tensor once) and the fraction of the HBM peak they amount to."""
+    """The other configurations in the same run: the height-bin sweep (fp32 forward on the 200 x 200 grid with
+    4, 8, 12 and 16 bins, the reference's headline experiment, tools/profile_latency.py:193-330), high-resolution
+    inference (bf16, forward) and training size (fp16, forward and backward), Laplace depth; event-timed calls,
+    compulsory bytes (every operand tensor once) and the fraction of the HBM peak they amount to."""
     got = {}
-    for name, with_backward in (("cfg4_hires", False), ("cfg5_train", True)):
-        w = WORKLOADS[name]
+    jobs = [(f"cfg3_zsweep_z{z}", WORKLOADS["cfg3_zsweep"].with_z(z), False) for z in (4, 8, 12, 16)]
+    jobs += [("cfg4_hires", WORKLOADS["cfg4_hires"], False), ("cfg5_train", WORKLOADS["cfg5_train"], True)]
+    for name, w, with_backward in jobs:
         r = Runner(w, "laplace", backward_mode=backward_mode)
         ms, fwd, bwd = time_steps(r, steps, warmup, with_backward)
         fb, bb = algorithmic_bytes(w, r.model, False), algorithmic_bytes(w, r.model, True)
@@ -358,8 +367,10 @@ def other_workloads(steps: int, warmup: int, backward_mode: int):
                                "frac_hbm": bb / b_ms / 1e6 / HBM_PEAK_GBS}
             rec["ms_per_step_fwd_bwd"] = ms
             rec["frac_hbm_fwd_bwd"] = (fb + bb) / ms / 1e6 / HBM_PEAK_GBS
-        c_ms, c_bytes = time_cached_forward(r, steps, warmup)
-        rec["forward_cached_geometry"] = {"ms": c_ms, "frac_hbm": fb / c_ms / 1e6 / HBM_PEAK_GBS, "cache_bytes": c_bytes}
+        if not name.startswith("cfg3"):
+            c_ms, c_bytes = time_cached_forward(r, steps, warmup)
+            rec["forward_cached_geometry"] = {"ms": c_ms, "frac_hbm": fb / c_ms / 1e6 / HBM_PEAK_GBS, "cache_bytes": c_bytes}
+        r.forward()
         rec["kept_samples"] = int(r.counts.sum().item())
         got[name] = rec
         del r
@@ -548,7 +559,11 @@ def main():
         "roofline": {"bound": "hbm", "kernel": f"{dominant} pass = " + " + ".join(k_names),
                      "dominant_kernel": top, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic[dominant] if traffic else None,
-                     "traffic_source": traffic["source"] if traffic else None, "algorithmic_bytes": k_bytes,
+                     "traffic_source": traffic["source"] if traffic else None,
+                     # the commit whose kernels the counters were collected on, and those kernels
+                     "traffic_commit": traffic.get("commit") if traffic else None,
+                     "traffic_kernels": traffic.get("kernels") if traffic else None,
+                     "algorithmic_bytes": k_bytes,
                      "kernel_ms": k_ms,
                      "forward": {"algorithmic_bytes": fb, "kernel_ms": fwd_k_ms,
                                  "frac": fb / fwd_k_ms / 1e6 / HBM_PEAK_GBS if fwd_k_ms else None}},

@@ -921,7 +921,8 @@ int fbev_backward_gather_static(const fbev_problem *p, const float *grad_out, co
     if (rc != FBEV_OK) return rc;
     // the per-kernel timers create HIP events: not in a call that promises to allocate nothing
     if (prof::enabled.load(std::memory_order_relaxed)) return FBEV_ERR_UNSUPPORTED;
-    // fixed segments only (three launches): the scratch array must hold the worst case of one pair per sample
+    // the scratch array must hold the worst case of one pair per sample (fixed segments, three launches, where a
+    // segment then has room for four pairs or more; the counted layout, which allocates nothing either, otherwise)
     const uint64_t max_pairs = fbev_backward_max_pairs(p);
     if (max_pairs >= (1ull << 31) || ws_index_bytes(p) + (size_t)max_pairs * sizeof(Pair) > (size_t)FBEV_STATIC_SCRATCH_BYTES)
         return FBEV_ERR_TOO_LARGE;

@@ -62,14 +62,24 @@ def _pair_capacity(batch: int, cams: int, grid) -> int:
 
 # Persistent inverse-map workspaces, one per (device, stream, problem shape, depth model): prepared
 # once, then every backward of that shape on that stream is two launches and allocates nothing.  The
-# few most recently used are kept (FLASHBEV_WORKSPACES, default 4; 0 switches them off and every
-# call takes its workspace from the caching allocator instead).
+# few most recently used are kept: at most FLASHBEV_WORKSPACES of them (default 4; 0 switches them off
+# and every call takes its workspace from the caching allocator instead) and at most
+# FLASHBEV_WORKSPACE_CACHE_MB in total (default 4096; this memory is not the caching allocator's to
+# hand out again, so torch.cuda.empty_cache() does not return it: release_workspaces() does).
+# A backward that runs while its stream is being captured into a graph leaves the cache alone and
+# takes a per-call workspace, which then comes from the graph's own memory pool: a graph must not
+# bake in a pointer that a later eviction or release_workspaces() frees, nor record the one-off
+# preparation of a workspace as something to replay.
 _workspaces: "collections.OrderedDict" = collections.OrderedDict()
 
 
 def release_workspaces() -> None:
     """Drop the persistent backward workspaces kept so far (they are prepared again on demand)."""
     _workspaces.clear()
+
+
+def _capturing() -> bool:
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
 
 
 def _stream_id(device) -> int:
@@ -79,7 +89,7 @@ def _stream_id(device) -> int:
 def _persistent_workspace(ext, depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
                           depth_distribution):
     keep = int(os.environ.get("FLASHBEV_WORKSPACES", "4"))
-    if keep <= 0:
+    if keep <= 0 or _capturing():
         return None, None
     key = (image_feats.device.index, _stream_id(image_feats.device),
            tuple(image_feats.shape), depth_params.shape[-1], tuple(grid_t.tolist()), int(depth_distribution))
@@ -88,12 +98,14 @@ def _persistent_workspace(ext, depth_params, image_feats, projection_matrices, f
         nbytes = ext.backward_workspace_bytes(depth_params, image_feats, projection_matrices, fs_host, image_t,
                                               grid_t, int(depth_distribution))
         limit_mb = float(os.environ.get("FLASHBEV_WORKSPACE_MB", "16384"))
-        if nbytes == 0 or nbytes > limit_mb * 2 ** 20:
+        total_mb = float(os.environ.get("FLASHBEV_WORKSPACE_CACHE_MB", "4096"))
+        if nbytes == 0 or nbytes > min(limit_mb, total_mb) * 2 ** 20:
             return None, None
         ws = ext.prepare_backward_workspace(depth_params, image_feats, projection_matrices, fs_host, image_t,
                                             grid_t, int(depth_distribution))
         _workspaces[key] = ws
-        while len(_workspaces) > keep:
+        # the least recently used go first, until both the count and the total size fit
+        while len(_workspaces) > keep or sum(t.numel() for t in _workspaces.values()) > total_mb * 2 ** 20:
             _workspaces.popitem(last=False)
     else:
         _workspaces.move_to_end(key)
@@ -169,7 +181,7 @@ def _check_feature_size(feature_size, cameras: int, H: int, W: int):
             if notes.get("feature_size_ok") == (H, W):
                 return
     else:
-        vals = [int(v) for row in feature_size for v in (row if hasattr(row, "__iter__") else [row])]
+        vals = [int(v) for v in np.asarray(feature_size).reshape(-1)]       # any nesting: [B][N][2], [B*N][2], flat
         if len(vals) != 2 * cameras:
             raise ValueError(f"feature_size must hold (H, W) for each of {cameras} cameras")
     if vals[0::2] != [H] * cameras or vals[1::2] != [W] * cameras:
@@ -204,6 +216,32 @@ def _feature_size_table(cameras: int, H: int, W: int):
     return torch.tensor([H, W], dtype=torch.int32).repeat(cameras)
 
 
+class GeometryCache:
+    """What ``build_geometry_cache`` returns: the lists (``data``, an opaque uint8 device tensor) together with what
+    they were built from, so that a forward handed the wrong cache raises on the host instead of pooling the wrong
+    texels: the matrices tensor (its storage address, version counter and shape -- an in-place update or another
+    tensor invalidates the cache, equal values in a new tensor do too: rebuild then), the feature-map and image
+    sizes, the grid, the region of interest and epsilon."""
+    __slots__ = ("data", "matrices", "sizes")
+
+    def __init__(self, data, projection_matrices, sizes):
+        self.data = data
+        self.matrices = self._identity(projection_matrices)
+        self.sizes = sizes
+
+    @staticmethod
+    def _identity(t):
+        return (t.data_ptr(), t._version, tuple(t.shape), t.dtype, t.device)
+
+    def check(self, projection_matrices, sizes) -> None:
+        if self._identity(projection_matrices) != self.matrices:
+            raise RuntimeError("geometry_cache was built from other projection matrices (another tensor, or this one "
+                               "was modified since): rebuild it with build_geometry_cache")
+        if sizes != self.sizes:
+            raise RuntimeError(f"geometry_cache was built for (feature map, image, grid, region, epsilon) = {self.sizes}, "
+                               f"this call has {sizes}: rebuild it with build_geometry_cache")
+
+
 class FlashBEVPool(torch.autograd.Function):
     """Fused projection + depth weighting + bilinear sampling + reduction over cameras and
     height bins.  Returns BEV features [B, Y, X, C] in float32."""
@@ -223,6 +261,7 @@ class FlashBEVPool(torch.autograd.Function):
             image_feats = image_feats.float()
         depth_params = depth_params.contiguous()
         image_feats = image_feats.contiguous()
+        matrices_given = projection_matrices
         projection_matrices = projection_matrices.contiguous().float()
         if reduction not in ("mean", "sum"):
             raise ValueError(f"reduction must be 'mean' or 'sum', got {reduction!r}")
@@ -239,6 +278,11 @@ class FlashBEVPool(torch.autograd.Function):
         image = _host_values(image_size, 2, "image_size", int)
         roi = _host_values(roi_range, 6, "roi_range", float)
         image_t, grid_t, roi_t, vmin, vsize = _host_arguments(grid, image, roi)
+        if isinstance(geometry_cache, GeometryCache):
+            # compared on the host, without a synchronisation (the kernel's own check of the cache's header, which
+            # answers a mismatch with NaN, stays behind this as the last line of defence)
+            geometry_cache.check(matrices_given, ((H, W), image, grid, tuple(np.float32(roi).tolist()), float(epsilon)))
+            geometry_cache = geometry_cache.data
 
         # feature_size repeats the feature tensor's (H, W) per camera: checked (a device tensor is
         # read once per object), then the extension gets a host table built from the shape
@@ -346,22 +390,24 @@ class _NoGrad:
 
 
 def build_geometry_cache(projection_matrices, feature_size, image_size, roi_range, grid_size, epsilon=1e-6):
-    """Per-cell lists of the samples in view for one calibration and grid, as an opaque uint8 tensor
+    """Per-cell lists of the samples in view for one calibration and grid, as a ``GeometryCache``
     for ``flash_bevpool(..., geometry_cache=...)``.  Worth building when ``projection_matrices``
     repeat from call to call (a fixed rig at inference); it must be rebuilt whenever the matrices,
     the feature-map or image size, the grid, the region of interest or ``epsilon`` change: a forward given
-    a cache that was built for other sizes or another region fills its output with NaN; a change of the
-    matrices alone goes unnoticed.  ``feature_size`` is (H, W) of the feature maps (a pair, or the operator's [B,N,2]
+    a cache that was built from another matrices tensor (or one modified in place since), other sizes or
+    another region raises.  (The bare ``.data`` tensor is accepted too; then only the kernel's own check of the sizes
+    and the region stands, which fills the output with NaN, and a change of the matrices goes unnoticed.)  ``feature_size`` is (H, W) of the feature maps (a pair, or the operator's [B,N,2]
     tensor).  Size: 16 bytes per (cell, camera, height bin) sample slot."""
     ext = load_ext()
     if isinstance(feature_size, torch.Tensor):
         fs = feature_size.reshape(-1).tolist() if feature_size.device.type == "cpu" else _device_values(feature_size)
     else:
-        fs = [int(v) for row in feature_size for v in (row if hasattr(row, "__iter__") else [row])]
+        fs = [int(v) for v in np.asarray(feature_size).reshape(-1)]
     H, W = int(fs[0]), int(fs[1])
     grid = _host_values(grid_size, 3, "grid_size", int)
     image = _host_values(image_size, 2, "image_size", int)
     roi = _host_values(roi_range, 6, "roi_range", float)
     vmin, vsize = voxel_geometry(roi, grid)
-    return ext.build_geometry_cache(projection_matrices.contiguous().float(), H, W, image[0], image[1], list(grid),
+    data = ext.build_geometry_cache(projection_matrices.contiguous().float(), H, W, image[0], image[1], list(grid),
                                     vmin, vsize, float(epsilon))
+    return GeometryCache(data, projection_matrices, ((H, W), image, grid, tuple(np.float32(roi).tolist()), float(epsilon)))

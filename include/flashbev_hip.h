@@ -210,7 +210,10 @@ int fbev_backward_gather_stored(const fbev_problem *p, const float *grad_out, co
  * no counterpart in the reference; it is for callers that cannot allocate device memory: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call makes no
  * hipMalloc / hipFree and calls no allocating library routine; inputs and outputs are the caller's,
- * as in fbev_backward_gather, and the results are the same (fixed segments, three launches).
+ * as in fbev_backward_gather, and the results are the same (fixed segments and three launches where a
+ * (texel, replica) segment of the worst-case layout holds four pairs or more, the counted layout otherwise).
+ * The first call on a device also asks the runtime for the array's address on that device and for the
+ * kernels' register counts (hipGetSymbolAddress, hipFuncGetAttributes): make that call outside a graph capture.
  * Limits: the worst-case workspace, fbev_backward_workspace_bytes(p, fbev_backward_max_pairs(p)),
  * must fit the scratch array, else FBEV_ERR_TOO_LARGE (128x128x8 cells x 6 cameras on a 16x44 map
  * needs 25.8 MB); with the per-kernel timers enabled (fbev_profile_enable), which create events,

@@ -146,6 +146,60 @@ def test_forward_and_backward_replay_from_a_hip_graph():
 
 
 @pytest.mark.gpu
+def test_a_captured_backward_keeps_clear_of_the_workspace_cache():
+    """A backward captured on an explicit stream, after eager steps on that stream have put a persistent workspace
+    for it into the cache: the captured call must not bake that workspace's pointer in (the cache may drop it at
+    any time) nor record a workspace's one-off preparation.  The cache is emptied after the capture, memory is
+    churned, and every replay still reproduces the eager gradients."""
+    import flashbev_amd
+    from flashbev_amd import flash_bevpool
+    from flashbev_amd.workloads import WORKLOADS, make_inputs
+    import sys
+    op = sys.modules["flashbev_amd.flash_bevpool"]
+
+    w = WORKLOADS["cfg2_surround"]
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    feats = x["image_feats"].clone().requires_grad_(True)
+    depth = x["depth_params"].clone().requires_grad_(True)
+    kw = dict(projection_matrices=x["projection_matrices"], feature_size=x["feature_size"],
+              image_size=list(w.image_hw), roi_range=list(w.roi_range), grid_size=list(w.grid_size),
+              depth_distribution=1, depth_weight_threshold=1e-6)
+
+    def step():
+        feats.grad = depth.grad = None
+        out = flash_bevpool(image_feats=feats, depth_params=depth, **kw)
+        out.backward(x["grad_out"])
+        return out
+
+    flashbev_amd.release_workspaces()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(3):
+            step()
+        want_f, want_d = feats.grad.clone(), depth.grad.clone()
+    torch.cuda.synchronize()
+    cached = dict(op._workspaces)
+    assert len(cached) == 1                         # the eager steps on this stream made one
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s):
+        step()
+    assert dict(op._workspaces).keys() == cached.keys()       # the capture neither added nor evicted
+    flashbev_amd.release_workspaces()
+    del cached
+    torch.cuda.empty_cache()
+    junk = [torch.full((8 << 20,), 7.0, device="cuda") for _ in range(4)]       # reuse what was freed
+    for i in range(3):
+        feats.grad.fill_(float("nan")); depth.grad.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.allclose(feats.grad, want_f, rtol=1e-4, atol=1e-5), f"replay {i}: d_feats differs"
+        assert torch.allclose(depth.grad, want_d, rtol=1e-4, atol=1e-5), f"replay {i}: d_depth differs"
+        assert all(bool((t == 7.0).all()) for t in junk), f"replay {i} wrote into memory it does not own"
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dist,channels", [(0, 80), (1, 80), (1, 13)])
 def test_interval_pooling_baseline_matches_the_oracle(dist, channels):
     """sampling_vt_pillarpool_fused on sample lists built from the oracle's own geometry equals

@@ -222,8 +222,23 @@ def test_operator_on_cached_geometry():
     assert torch.equal(outs[0], outs[1])
     assert torch.allclose(grads[0][0].float(), grads[1][0].float(), rtol=1e-3, atol=1e-4)
     assert torch.allclose(grads[0][1].float(), grads[1][1].float(), rtol=1e-3, atol=1e-4)
-    with pytest.raises(RuntimeError, match="inconsistent"):
+    # a cache that does not belong to the call is refused on the host: another grid, another region of
+    # interest, another matrices tensor (equal values included), the same tensor modified in place
+    with pytest.raises(RuntimeError, match="rebuild it"):
         flash_bevpool(image_feats=x["image_feats"], depth_params=x["depth_params"], geometry_cache=cache,
+                      **dict(args, grid_size=(48, 48, 6)))
+    with pytest.raises(RuntimeError, match="rebuild it"):
+        flash_bevpool(image_feats=x["image_feats"], depth_params=x["depth_params"], geometry_cache=cache,
+                      **dict(args, roi_range=[v * 0.5 for v in w.roi_range]))
+    with pytest.raises(RuntimeError, match="other projection matrices"):
+        flash_bevpool(image_feats=x["image_feats"], depth_params=x["depth_params"], geometry_cache=cache,
+                      **dict(args, projection_matrices=x["projection_matrices"].clone()))
+    x["projection_matrices"].mul_(1.0)
+    with pytest.raises(RuntimeError, match="other projection matrices"):
+        flash_bevpool(image_feats=x["image_feats"], depth_params=x["depth_params"], geometry_cache=cache, **args)
+    # the bare tensor is still accepted; there the library's own check of the sizes refuses another grid
+    with pytest.raises(RuntimeError, match="inconsistent"):
+        flash_bevpool(image_feats=x["image_feats"], depth_params=x["depth_params"], geometry_cache=cache.data,
                       **dict(args, grid_size=(48, 48, 6)))
 
 

@@ -14,17 +14,26 @@ pytestmark = pytest.mark.gpu
 MODEL = {0: "parametric", 1: "parametric", 2: "categorical"}
 
 
-def static_backward(x, w, dist, overwrite):
+def static_backward(x, w, dist, overwrite, check_memory=False):
     p = U.problem_for(x, w, dist)
     dev = x["image_feats"].device
     fill = float("nan") if overwrite else 0.0
     dd = torch.full(x["depth_params"].shape, fill, dtype=torch.float32, device=dev)
     df = torch.full(x["image_feats"].shape, fill, dtype=torch.float32, device=dev)
-    capi.check(capi.backward_gather_static(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
-                                           x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(),
-                                           dd.data_ptr(), df.data_ptr(), torch.cuda.current_stream().cuda_stream,
-                                           accumulate=not overwrite), "fbev_backward_gather_static")
+    args = (p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(), x["image_feats"].data_ptr(),
+            x["projection_matrices"].data_ptr(), dd.data_ptr(), df.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    capi.check(capi.backward_gather_static(*args, accumulate=not overwrite), "fbev_backward_gather_static")
     torch.cuda.synchronize()
+    if check_memory:
+        # what the entry point exists for: once a first call on the device has resolved the scratch array's
+        # address, a call takes no device memory (the driver's count of free bytes stays where it was)
+        keep = (dd.clone(), df.clone())
+        free_before = torch.cuda.mem_get_info()[0]
+        capi.check(capi.backward_gather_static(*args, accumulate=not overwrite), "fbev_backward_gather_static")
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        if overwrite:
+            dd, df = keep
     return dd, df
 
 
@@ -37,7 +46,7 @@ def test_static_scratch_backward_matches_the_workspace_backward_on_two_calls_in_
         p = U.problem_for(x, w, dist)
         assert capi.backward_workspace_bytes(p, capi.backward_max_pairs(p)) <= capi.static_scratch_bytes()
         want_dd, want_df = U.capi_backward(x, w, dist, mode="gather")
-        dd, df = static_backward(x, w, dist, overwrite)
+        dd, df = static_backward(x, w, dist, overwrite, check_memory=overwrite)
         # same kernels, same layout; only the order in which samples claimed their places differs
         # from call to call, and with it the order of the fp32 sums: the stated tolerance
         for got, ref, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
