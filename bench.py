@@ -78,7 +78,7 @@ class Runner:
     """Pre-allocated buffers and the four queued operations of one step."""
 
     def __init__(self, w, depth_name: str, device: str = "cuda:0", backward_mode: int = 0, persistent: bool = True,
-                 sample_store: bool = True):
+                 sample_store: bool = True, workspace_layout=None):
         self.w = w
         self.backward_mode = backward_mode
         self.dist, self.model = DIST_OF[depth_name]
@@ -105,11 +105,21 @@ class Runner:
         self.stored_by_forward = False
         # the inverse map's workspace, prepared once (what the autograd operator keeps per shape);
         # persistent=False takes a fresh workspace from the caching allocator in every call instead
+        # (laid out as the operator lays it out: segments sized by the geometry where room for every sample would
+        # take more than 64 MB, segments of one common capacity below that)
         self.workspace = None
+        self.workspace_layout = 1
         if persistent and backward_mode in (0, 2):
+            from flashbev_amd.flash_bevpool import _SIZED_FROM_BYTES, _workspace_layout
             nbytes = self.ext.backward_workspace_bytes(x["depth_params"], x["image_feats"], x["projection_matrices"],
                                                        x["feature_size"], x["image_size"], x["grid_size"], self.dist)
-            if nbytes:
+            want = _workspace_layout() if workspace_layout is None else workspace_layout
+            if nbytes and (want == "sized" or (want == "auto" and nbytes > _SIZED_FROM_BYTES)):
+                self.workspace = self.ext.prepare_sized_backward_workspace(
+                    x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
+                    x["image_size"], x["grid_size"], self.dist, list(self.vmin), list(self.vsize), self.eps)
+                self.workspace_layout = 2
+            elif nbytes:
                 self.workspace = self.ext.prepare_backward_workspace(
                     x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
                     x["image_size"], x["grid_size"], self.dist)
@@ -137,7 +147,8 @@ class Runner:
             x["grad_out"], x["depth_params"], x["image_feats"], x["projection_matrices"], x["feature_size"],
             x["image_size"], x["roi_range"], x["grid_size"], self.d_depth, self.d_feats, self.out.numel(),
             self.dist, self.eps, self.thr, w.depth_range[0], w.depth_range[1], 0, self.backward_mode, -1,
-            self.counts, False, self.workspace, self.store if self.stored_by_forward else None, list(self.vsize))
+            self.counts, False, self.workspace, self.store if self.stored_by_forward else None, list(self.vsize),
+            self.workspace_layout)
 
 
 # Untimed steps of the workload itself, run for this many milliseconds before the warm-up steps of every
@@ -372,6 +383,10 @@ def other_workloads(steps: int, warmup: int, backward_mode: int):
             rec["forward_cached_geometry"] = {"ms": c_ms, "frac_hbm": fb / c_ms / 1e6 / HBM_PEAK_GBS, "cache_bytes": c_bytes}
         r.forward()
         rec["kept_samples"] = int(r.counts.sum().item())
+        if with_backward and r.workspace is not None:
+            rec["backward_workspace"] = {"bytes": r.workspace.numel(),
+                                         "layout": "segments sized by the geometry" if r.workspace_layout == 2
+                                         else "segments of one common capacity"}
         got[name] = rec
         del r
         torch.cuda.empty_cache()

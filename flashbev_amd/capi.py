@@ -15,7 +15,7 @@ FBEV_F32, FBEV_F16, FBEV_BF16 = 0, 1, 2
 FBEV_GAUSSIAN, FBEV_LAPLACE, FBEV_CATEGORICAL = 0, 1, 2
 FBEV_REDUCE_MEAN, FBEV_REDUCE_SUM = 0, 1
 
-EXPORTS = ("fbev_forward", "fbev_sample_store_bytes", "fbev_forward_store", "fbev_backward_gather_stored", "fbev_geometry_cache_bytes", "fbev_geometry_cache_build", "fbev_forward_cached", "fbev_backward", "fbev_backward_gather", "fbev_backward_gather_static",
+EXPORTS = ("fbev_forward", "fbev_backward_sized_workspace_bytes", "fbev_backward_sized_total_offset", "fbev_backward_workspace_init_sized", "fbev_backward_gather_sized", "fbev_sample_store_bytes", "fbev_forward_store", "fbev_backward_gather_stored", "fbev_geometry_cache_bytes", "fbev_geometry_cache_build", "fbev_forward_cached", "fbev_backward", "fbev_backward_gather", "fbev_backward_gather_static",
            "fbev_static_scratch_bytes", "fbev_backward_persistent_workspace_bytes", "fbev_backward_workspace_init",
            "fbev_backward_gather_persistent", "fbev_backward_columns",
            "fbev_backward_columns_workspace_bytes", "fbev_backward_max_pairs",
@@ -56,6 +56,14 @@ def load() -> ctypes.CDLL:
         vp, pp = ctypes.c_void_p, ctypes.POINTER(FbevProblem)
         lib.fbev_forward.argtypes = [pp, vp, vp, vp, vp, vp, vp]
         lib.fbev_forward.restype = ctypes.c_int
+        lib.fbev_backward_sized_workspace_bytes.argtypes = [pp, ctypes.c_uint64]
+        lib.fbev_backward_sized_workspace_bytes.restype = ctypes.c_size_t
+        lib.fbev_backward_sized_total_offset.argtypes = [pp]
+        lib.fbev_backward_sized_total_offset.restype = ctypes.c_size_t
+        lib.fbev_backward_workspace_init_sized.argtypes = [pp, vp, vp, ctypes.c_size_t, vp]
+        lib.fbev_backward_workspace_init_sized.restype = ctypes.c_int
+        lib.fbev_backward_gather_sized.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_int, vp, ctypes.c_size_t, vp]
+        lib.fbev_backward_gather_sized.restype = ctypes.c_int
         lib.fbev_sample_store_bytes.argtypes = [pp]
         lib.fbev_sample_store_bytes.restype = ctypes.c_size_t
         lib.fbev_forward_store.argtypes = [pp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp]
@@ -178,7 +186,7 @@ def backward_gather_stored(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, fe
                                               _p(proj_ptr), _p(cell_count_ptr), _p(store_ptr),
                                               ctypes.c_size_t(int(store_bytes)), _p(d_depth_ptr), _p(d_feats_ptr),
                                               int(bool(accumulate)), _p(workspace_ptr),
-                                              ctypes.c_size_t(int(workspace_bytes)), int(bool(persistent)), _p(stream))
+                                              ctypes.c_size_t(int(workspace_bytes)), int(persistent), _p(stream))
 
 
 def geometry_cache_bytes(p: FbevProblem) -> int:
@@ -237,6 +245,29 @@ def backward_gather_persistent(p: FbevProblem, grad_out_ptr: int, depth_ptr: int
                                                   _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr),
                                                   int(bool(accumulate)), _p(workspace_ptr),
                                                   ctypes.c_size_t(int(workspace_bytes)), _p(stream))
+
+
+def backward_sized_workspace_bytes(p: FbevProblem, pair_capacity: int) -> int:
+    return int(load().fbev_backward_sized_workspace_bytes(ctypes.byref(p), ctypes.c_uint64(int(pair_capacity))))
+
+
+def backward_sized_total_offset(p: FbevProblem) -> int:
+    return int(load().fbev_backward_sized_total_offset(ctypes.byref(p)))
+
+
+def backward_workspace_init_sized(p: FbevProblem, proj_ptr: int, workspace_ptr: int, workspace_bytes: int,
+                                  stream: int = 0) -> int:
+    return load().fbev_backward_workspace_init_sized(ctypes.byref(p), _p(proj_ptr), _p(workspace_ptr),
+                                                     ctypes.c_size_t(int(workspace_bytes)), _p(stream))
+
+
+def backward_gather_sized(p: FbevProblem, grad_out_ptr: int, depth_ptr: int, feats_ptr: int, proj_ptr: int,
+                          d_depth_ptr: Optional[int], d_feats_ptr: Optional[int], workspace_ptr: int,
+                          workspace_bytes: int, stream: int = 0, accumulate: bool = True) -> int:
+    """fbev_backward_gather_persistent on a workspace whose segments backward_workspace_init_sized sized."""
+    return load().fbev_backward_gather_sized(ctypes.byref(p), _p(grad_out_ptr), _p(depth_ptr), _p(feats_ptr),
+                                             _p(proj_ptr), _p(d_depth_ptr), _p(d_feats_ptr), int(bool(accumulate)),
+                                             _p(workspace_ptr), ctypes.c_size_t(int(workspace_bytes)), _p(stream))
 
 
 def static_scratch_bytes() -> int:

@@ -60,7 +60,9 @@ __global__ __launch_bounds__(256) void fbev_fill_zero_kernel(int *a, long long n
 
 // Count, per (first-corner texel, replica), the samples that will contribute: phase A alone, with
 // exactly the decisions the cell pass takes later (same code, same inputs).
-template <typename T>
+// VIEW: count the samples in view (no depth model, no threshold) per fixed segment instead: the capacities of
+// segments sized by the geometry.
+template <typename T, bool VIEW = false>
 __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_count_kernel(KParams k, const T *__restrict__ depth,
                                                                          const float *__restrict__ proj,
                                                                          int *__restrict__ counts) {
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_count_kernel(KPara
         const int q0 = (blk * k.waves + wave) * cells_per_wave + r * k.slots_a;
         if (q0 >= k.padded_cells) break;
         const int n_cand = phase_a_candidates<false>(k, L, q0, lane);     // group boundaries are not needed
-        phase_a_samples<0, T, kModeCount>(k, L, depth, b, lane, 0, n_cand, nullptr, counts, 0);      // no entries: no pool
+        phase_a_samples<0, T, VIEW ? kModeCountView : kModeCount>(k, L, depth, b, lane, 0, n_cand, nullptr, counts, 0);      // no entries: no pool
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -155,6 +157,15 @@ __global__ __launch_bounds__(1024) void fbev_scan_sums_kernel(int *v, int n) {
     }
 }
 
+// The table of segments sized by the geometry: absolute start and capacity of every segment, from the
+// capacities, their prefix sums within chunks of 4096 and the chunks' prefix sums.
+__global__ __launch_bounds__(256) void fbev_segment_table_kernel(long long n, const int *__restrict__ cap,
+                                                                 const int *__restrict__ off,
+                                                                 const int *__restrict__ prefix, int2 *__restrict__ tab) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) tab[i] = make_int2(prefix[i >> kScanChunkBits] + off[i], cap[i]);
+}
+
 // Cell pass of the backward.  FILL = 0: scatter with atomics.  FILL = 1: write pairs (inverse
 // map); FILL = 2: the same with one claim per run of samples on one texel; FILL = 3: write pairs for the
 // samples the forward stored (`store`, with the forward's per-cell counts in `count`) instead of
@@ -166,7 +177,8 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
     KParams k, const float *__restrict__ grad_out, const T *__restrict__ depth, const T *__restrict__ feats,
     const float *__restrict__ proj, float *__restrict__ d_depth, float *__restrict__ d_feats,
     const int *__restrict__ chunk_prefix, int *__restrict__ cursor, Pair *__restrict__ pairs, int pair_cap,
-    int *epoch, int set_stride, const float *__restrict__ count = nullptr, const float4 *__restrict__ store = nullptr) {
+    int *epoch, int set_stride, const float *__restrict__ count = nullptr, const float4 *__restrict__ store = nullptr,
+    const SegTable segs = SegTable{nullptr}) {
     extern __shared__ float4 smem[];
     constexpr int EF4 = 2;
     constexpr bool STORED = FILL == 3;
@@ -268,11 +280,11 @@ __global__ __launch_bounds__(kWave *kWavesPerBlock) void fbev_backward_cells_ker
         }
         if (STORED)
             phase_a_stored(k, L, count, store + ((size_t)b * k.padded_cells + q0) * k.NZ * 2, b, q0, lane, chunk_prefix,
-                           cursor, pair_cap);
+                           cursor, pair_cap, segs);
         else
             phase_a_samples<EF4, T, FILL == 2 ? kModeFillRuns : (FILL ? kModeFill : kModeScatter)>(
                 k, L, depth, b, lane, BATCHED ? L.gcand[g0] : 0, BATCHED ? L.gcand[g0 + step] : n_cand, chunk_prefix, cursor,
-                pair_cap);
+                pair_cap, nullptr, segs);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         for (int grp = g0; grp < g0 + step; ++grp) {

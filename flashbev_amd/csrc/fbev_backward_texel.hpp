@@ -34,11 +34,13 @@ constexpr int kTexelSegs = 4 * kFixedReplicas;   // lists of a texel with fixed 
 //              cannot file (a full segment) or does not file (a depth gradient that does not ride on
 //              the pairs) it adds here with atomics; the texel pass of a texel that sees a full
 //              segment, the only texels such samples reach, takes its rows from here and clears them.
+//   segs       segments sized by the geometry (see SegTable), or all null for segments of one common capacity.
 struct Persist {
     int *epoch;
     int *sets;
     int set_stride;
     float *ovf_depth, *ovf_feats;
+    SegTable segs;
 };
 
 template <int VEC, int WAVES>
@@ -97,6 +99,13 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             // fixed segments of pair_cap pairs; seg_end holds how many were claimed
             const int i = q * kFixedReplicas + (e >> 2);
             my_lo = i * pair_cap;
+            int room = pair_cap;
+            if (ps.segs.tab != nullptr) {
+                // (a segment that would reach past the pair array holds what fits: the rest was added with atomics)
+                const int2 seg = ps.segs.tab[i];
+                my_lo = seg.x;
+                room = max(min(seg.y, pair_cap - my_lo), 0);
+            }
             int claimed;
             if (persistent) {
                 const int in_first = ps.sets[i], in_second = ps.sets[ps.set_stride + i];
@@ -104,8 +113,8 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             } else {
                 claimed = seg_end[i];
             }
-            spilled = claimed > pair_cap;
-            my_len = max(min(claimed, pair_cap), 0);
+            spilled = claimed > room;
+            my_len = max(min(claimed, room), 0);
         }
     }
     if (persistent && threadIdx.x == 0 && blockIdx.y == 0) {

@@ -336,7 +336,8 @@ int launch_columns(const Plan &pl, const ColParams &cp, size_t lds, const float 
 template <typename T, int VEC, int FILL>
 int launch_cells(const Plan &pl, const float *go, const void *depth, const void *feats, const float *proj,
                  float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap, hipStream_t st,
-                 int *epoch = nullptr, int set_stride = 0, const float *count = nullptr, const float4 *store = nullptr) {
+                 int *epoch = nullptr, int set_stride = 0, const float *count = nullptr, const float4 *store = nullptr,
+                 SegTable segs = SegTable{nullptr}) {
     dim3 grid(pl.k.n_blocks), block(kWave * pl.k.waves);
     const T *d = static_cast<const T *>(depth);
     const T *f = static_cast<const T *>(feats);
@@ -348,7 +349,7 @@ int launch_cells(const Plan &pl, const float *go, const void *depth, const void 
     auto launch = [&](auto kernel) {
         if (!lds_opt_in(kernel, lds)) return false;
         hipLaunchKernelGGL(kernel, grid, block, lds, st, pl.k, go, d, f, proj, dd, df, prefix, cursor, pairs, cap, epoch, set_stride,
-                           count, store);
+                           count, store, segs);
         return true;
     };
     auto pick = [&](auto cpl_tag) {
@@ -410,25 +411,25 @@ template <int FILL>
 int dispatch_cells(const fbev_problem *p, const Plan &pl, const float *go, const void *depth, const void *feats,
                    const float *proj, float *dd, float *df, const int *prefix, int *cursor, Pair *pairs, int cap,
                    hipStream_t st, int *epoch = nullptr, int set_stride = 0, const float *count = nullptr,
-                   const float4 *store = nullptr) {
+                   const float4 *store = nullptr, SegTable segs = SegTable{nullptr}) {
     switch (p->in_dtype) {
         case FBEV_F32:
-            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store)
-                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store);
+            return pl.vec == 4 ? launch_cells<float, 4, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store, segs)
+                               : launch_cells<float, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store, segs);
         case FBEV_F16:
-            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store)
-                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store);
+            return pl.vec == 8 ? launch_cells<__half, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store, segs)
+                               : launch_cells<__half, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store, segs);
         default:
-            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store)
-                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store);
+            return pl.vec == 8 ? launch_cells<bf16_raw, 8, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store, segs)
+                               : launch_cells<bf16_raw, 1, FILL>(pl, go, depth, feats, proj, dd, df, prefix, cursor, pairs, cap, st, epoch, set_stride, count, store, segs);
     }
 }
 
-template <typename T>
+template <typename T, bool VIEW = false>
 int launch_count(const Plan &pl, const void *depth, const float *proj, int *counts, hipStream_t st) {
-    if (!lds_opt_in(fbev_count_kernel<T>, pl.lds_count)) return FBEV_ERR_LAUNCH;
+    if (!lds_opt_in(fbev_count_kernel<T, VIEW>, pl.lds_count)) return FBEV_ERR_LAUNCH;
     prof::Scope timer(prof::kCount, st);
-    hipLaunchKernelGGL((fbev_count_kernel<T>), dim3(pl.k.n_blocks), dim3(kWave * pl.k.waves), pl.lds_count, st, pl.k,
+    hipLaunchKernelGGL((fbev_count_kernel<T, VIEW>), dim3(pl.k.n_blocks), dim3(kWave * pl.k.waves), pl.lds_count, st, pl.k,
                        static_cast<const T *>(depth), proj, counts);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
@@ -455,11 +456,17 @@ size_t ws_index_bytes(const fbev_problem *p) {
 //   [256 bytes: the two call counters][two sets of texels * kFixedReplicas claim counters]
 //   [a depth-gradient and a feature-gradient buffer of the workspace's own], each padded to 256 bytes,
 // then the pairs.  fbev_backward_workspace_init zero-fills all of it but the pairs, once.
+// A workspace whose segments are sized by the geometry (fbev_backward_workspace_init_sized) holds, between the
+// gradient buffers and the pairs, the table the kernels read (per segment its start in the pair array and its
+// capacity, the samples in view that claim there) and what it was made from: the capacities, their prefix sums
+// within scan chunks of 4096 segments, and per chunk the pairs before it, with the total behind the last chunk.
 struct PersistLayout {
     size_t sets, ovf_depth, ovf_feats, pairs;      // byte offsets
     long long set_stride;                          // ints between the two sets
+    size_t seg_tab, seg_cap, seg_off, seg_prefix;  // byte offsets of the tables (sized segments only)
+    long long seg_chunks;                          // scan chunks of the segment tables
 };
-PersistLayout persist_layout(const fbev_problem *p) {
+PersistLayout persist_layout(const fbev_problem *p, bool sized = false) {
     auto pad = [](size_t n) { return (n + 255) / 256 * 256; };
     const size_t texels = (size_t)texel_count(p);
     PersistLayout l;
@@ -468,6 +475,15 @@ PersistLayout persist_layout(const fbev_problem *p) {
     l.ovf_depth = l.sets + pad(2 * (size_t)l.set_stride * sizeof(int));
     l.ovf_feats = l.ovf_depth + pad(texels * p->depth_bins * sizeof(float));
     l.pairs = l.ovf_feats + pad(texels * p->channels * sizeof(float));
+    l.seg_tab = l.seg_cap = l.seg_off = l.seg_prefix = 0;
+    l.seg_chunks = (l.set_stride + (1ll << kScanChunkBits) - 1) >> kScanChunkBits;
+    if (sized) {
+        l.seg_tab = l.pairs;
+        l.seg_cap = l.seg_tab + pad((size_t)l.set_stride * sizeof(int2));
+        l.seg_off = l.seg_cap + pad((size_t)l.set_stride * sizeof(int));
+        l.seg_prefix = l.seg_off + pad((size_t)l.set_stride * sizeof(int));
+        l.pairs = l.seg_prefix + pad((size_t)(l.seg_chunks + 1) * sizeof(int));
+    }
     return l;
 }
 
@@ -520,8 +536,12 @@ int scratch_of_current_device(void **out) {
 
 int backward_gather_impl(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
                          const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
-                         size_t workspace_bytes, void *stream, bool persistent = false, const float *cell_count = nullptr,
+                         size_t workspace_bytes, void *stream, int ws_kind = 0, const float *cell_count = nullptr,
                          const void *store = nullptr, size_t store_bytes = 0) {
+    // ws_kind: 0 a per-call workspace, 1 a persistent one with segments of one common capacity, 2 a persistent
+    // one whose segments were sized by the geometry
+    if (ws_kind < 0 || ws_kind > 2) return FBEV_ERR_UNSUPPORTED;
+    const bool persistent = ws_kind != 0, sized = ws_kind == 2;
     int rc = validate(p, true);
     if (rc != FBEV_OK) return rc;
     rc = check_backward_args(p, grad_out, depth, feats, proj, d_depth, d_feats);
@@ -529,7 +549,7 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     if (!d_depth && !d_feats) return FBEV_OK;
     if (!workspace) return FBEV_ERR_NULL;
     if ((uintptr_t)workspace % 16) return FBEV_ERR_ALIGNMENT;
-    const PersistLayout lay = persist_layout(p);
+    const PersistLayout lay = persist_layout(p, sized);
     const size_t index_bytes = persistent ? lay.pairs : ws_index_bytes(p);
     if (workspace_bytes < index_bytes) return FBEV_ERR_SHAPE;
     // pair positions are 32-bit: every sample must be countable
@@ -548,7 +568,7 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
         // (where a claim counter may get hundreds of samples the claims go per run, which the stored samples do
         // not: such problems evaluate their samples again)
         const long long tx = texel_count(p);
-        const bool fixed_layout = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (tx * kFixedReplicas) >= kFixedMinSegment;
+        const bool fixed_layout = sized || ((uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (tx * kFixedReplicas) >= kFixedMinSegment);
         if (sample_count(p) / (fixed_layout ? tx * kFixedReplicas : counter_count(p)) >= kClaimRunsFrom) stored = false;
     }
     if (stored) {
@@ -563,7 +583,7 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     if (!stored) {
         // the cell pass in batches of several groups only where that does not cost occupancy
         const long long tx = texel_count(p);
-        const bool fixed_layout = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (tx * kFixedReplicas) >= kFixedMinSegment;
+        const bool fixed_layout = sized || ((uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (tx * kFixedReplicas) >= kFixedMinSegment);
         const bool runs = sample_count(p) / (fixed_layout ? tx * kFixedReplicas : counter_count(p)) >= kClaimRunsFrom;
         if (pl.k.batch_groups > 1 && !(runs ? cells_batch_pays<2>(p, pl) : cells_batch_pays<1>(p, pl))) {
             rc = make_plan(p, allow_vec, &pl, kCellPassWaves, 3, kMaxSlotLdsBytes, 1);
@@ -582,11 +602,14 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     // owns cap / (texels * kFixedReplicas) pair slots, and the counting pass and the prefix sums
     // are not needed.  (A texel that outgrows its segments falls back to atomics, like a full
     // pair array does.)  Smaller workspaces are packed exactly: count, scan, fill.
-    const bool fixed = (uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (texels * kFixedReplicas) >= kFixedMinSegment;
-    if (persistent && !fixed) return FBEV_ERR_SHAPE;      // a persistent workspace holds the worst case
-    const int seg_cap = fixed ? (int)(cap / (texels * kFixedReplicas)) : 0;
+    const bool fixed = sized || ((uint64_t)cap >= fbev_backward_max_pairs(p) && cap / (texels * kFixedReplicas) >= kFixedMinSegment);
+    if (persistent && !fixed) return FBEV_ERR_SHAPE;      // a persistent workspace holds the worst case, or sized segments
+    // (with sized segments the kernels compare positions with the whole array's capacity)
+    const int seg_cap = sized ? cap : (fixed ? (int)(cap / (texels * kFixedReplicas)) : 0);
     // what the two kernels get when the workspace is persistent: no zero-fill launch then
-    Persist ps = {nullptr, nullptr, 0, nullptr, nullptr};
+    Persist ps = {nullptr, nullptr, 0, nullptr, nullptr, SegTable{nullptr}};
+    if (sized)
+        ps.segs = SegTable{reinterpret_cast<const int2 *>(base + lay.seg_tab)};
     float *cells_dd = d_depth, *cells_df = d_feats;
     if (persistent) {
         ps.epoch = reinterpret_cast<int *>(base);
@@ -627,12 +650,12 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     const bool claim_runs = sample_count(p) / (fixed ? texels * kFixedReplicas : counters) >= kClaimRunsFrom;
     if (stored)
         rc = dispatch_cells<3>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs, cap_arg, st,
-                               ps.epoch, ps.set_stride, cell_count, static_cast<const float4 *>(store));
+                               ps.epoch, ps.set_stride, cell_count, static_cast<const float4 *>(store), ps.segs);
     else
     rc = claim_runs ? dispatch_cells<2>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs,
-                                        cap_arg, st, ps.epoch, ps.set_stride)
+                                        cap_arg, st, ps.epoch, ps.set_stride, nullptr, nullptr, ps.segs)
                     : dispatch_cells<1>(p, pl, grad_out, depth, feats, proj, cells_dd, cells_df, prefix_arg, cursor, pairs,
-                                        cap_arg, st, ps.epoch, ps.set_stride);
+                                        cap_arg, st, ps.epoch, ps.set_stride, nullptr, nullptr, ps.segs);
     if (rc != FBEV_OK) return rc;
 
     // texel pass: rows of grad_out are fp32, so 128-bit gathers need C % 4 == 0 and aligned rows
@@ -688,6 +711,50 @@ int workspace_init_impl(const fbev_problem *p, void *workspace, size_t workspace
     const PersistLayout lay = persist_layout(p);
     if (workspace_bytes < lay.pairs) return FBEV_ERR_SHAPE;
     return launch_zero(static_cast<int *>(workspace), (long long)(lay.pairs / sizeof(int)), nullptr, 0, nullptr, 0, st);
+}
+
+// Prepare a persistent workspace whose segments are sized by the geometry: zero-fill everything but the pairs,
+// count the samples in view per segment (no depth model: an upper bound of what any depth tensor and threshold
+// keep), and prefix-sum the counts into the segments' starts.
+int workspace_init_sized_impl(const fbev_problem *p, const float *proj, void *workspace, size_t workspace_bytes,
+                              hipStream_t st) {
+    int rc = validate(p, true);
+    if (rc != FBEV_OK) return rc;
+    if (!workspace || !proj) return FBEV_ERR_NULL;
+    if ((uintptr_t)workspace % 16 || (uintptr_t)proj % 4) return FBEV_ERR_ALIGNMENT;
+    if (sample_count(p) >= (1ll << 31) || counter_count(p) >= (1ll << 31)) return FBEV_ERR_TOO_LARGE;
+    const PersistLayout lay = persist_layout(p, true);
+    if (workspace_bytes < lay.pairs) return FBEV_ERR_SHAPE;
+    rc = launch_zero(static_cast<int *>(workspace), (long long)(lay.pairs / sizeof(int)), nullptr, 0, nullptr, 0, st);
+    if (rc != FBEV_OK) return rc;
+    fbev_problem q = *p;      // the samples in view depend on the geometry only
+    q.channels = 4; q.in_dtype = FBEV_F32; q.depth_distribution = FBEV_GAUSSIAN; q.depth_bins = 2;
+    q.reduction = FBEV_REDUCE_MEAN;
+    Plan pl;
+    rc = make_plan(&q, true, &pl, kCellPassWaves);
+    if (rc != FBEV_OK) return rc;
+    char *base = static_cast<char *>(workspace);
+    int *seg_cap = reinterpret_cast<int *>(base + lay.seg_cap), *seg_off = reinterpret_cast<int *>(base + lay.seg_off);
+    int *seg_prefix = reinterpret_cast<int *>(base + lay.seg_prefix);
+    rc = launch_count<float, true>(pl, nullptr, proj, seg_cap, st);
+    if (rc != FBEV_OK) return rc;
+    if (hipMemcpyAsync(seg_off, seg_cap, (size_t)lay.set_stride * sizeof(int), hipMemcpyDeviceToDevice, st) != hipSuccess)
+        return FBEV_ERR_LAUNCH;
+    {
+        prof::Scope timer(prof::kScanChunks, st);
+        hipLaunchKernelGGL(fbev_scan_chunks_kernel, dim3((unsigned)lay.seg_chunks), dim3(1024), 0, st, seg_off,
+                           lay.set_stride, seg_prefix);
+    }
+    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+    {
+        // (one entry more than there are chunks, zero so far: it receives the total)
+        prof::Scope timer(prof::kScanSums, st);
+        hipLaunchKernelGGL(fbev_scan_sums_kernel, dim3(1), dim3(1024), 0, st, seg_prefix, (int)lay.seg_chunks + 1);
+    }
+    if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
+    hipLaunchKernelGGL(fbev_segment_table_kernel, dim3((unsigned)((lay.set_stride + 255) / 256)), dim3(256), 0, st,
+                       lay.set_stride, seg_cap, seg_off, seg_prefix, reinterpret_cast<int2 *>(base + lay.seg_tab));
+    return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 
 }  // namespace
@@ -903,7 +970,30 @@ int fbev_backward_gather_persistent(const fbev_problem *p, const float *grad_out
                                     const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
                                     size_t workspace_bytes, void *stream) {
     return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
-                                workspace_bytes, stream, true);
+                                workspace_bytes, stream, 1);
+}
+
+size_t fbev_backward_sized_workspace_bytes(const fbev_problem *p, uint64_t pair_capacity) {
+    if (validate(p, true) != FBEV_OK) return 0;
+    return persist_layout(p, true).pairs + (size_t)pair_capacity * sizeof(Pair);
+}
+
+size_t fbev_backward_sized_total_offset(const fbev_problem *p) {
+    if (validate(p, true) != FBEV_OK) return 0;
+    const PersistLayout lay = persist_layout(p, true);
+    return lay.seg_prefix + (size_t)lay.seg_chunks * sizeof(int);
+}
+
+int fbev_backward_workspace_init_sized(const fbev_problem *p, const float *proj, void *workspace, size_t workspace_bytes,
+                                       void *stream) {
+    return workspace_init_sized_impl(p, proj, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int fbev_backward_gather_sized(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                               const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
+                                workspace_bytes, stream, 2);
 }
 
 int fbev_backward_gather_stored(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
@@ -912,7 +1002,7 @@ int fbev_backward_gather_stored(const fbev_problem *p, const float *grad_out, co
                                 int persistent, void *stream) {
     if (!store) return FBEV_ERR_NULL;
     return backward_gather_impl(p, grad_out, depth, feats, proj, d_depth, d_feats, accumulate, workspace,
-                                workspace_bytes, stream, persistent != 0, cell_count, store, store_bytes);
+                                workspace_bytes, stream, persistent, cell_count, store, store_bytes);
 }
 
 int fbev_backward_gather_static(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,

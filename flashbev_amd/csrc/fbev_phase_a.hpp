@@ -97,14 +97,33 @@ __device__ __forceinline__ WaveLds block_lds_setup(const KParams &k, float4 *sme
 //             words per kept sample in the slot of its cell (cells in the order of the tiled walk, N * gz entries
 //             per cell): the backward entry above with -1 in the fourth place (no pair position yet)
 enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeFillRuns = 4, kModeCache = 5,
-       kModeForwardStore = 6 };
+       kModeForwardStore = 6, kModeCountView = 7 };
+
+// Segments sized by the geometry (a persistent workspace prepared for one set of matrices): segment i =
+// (texel, replica) starts at tab[i].x in the pair array and has room for tab[i].y pairs, the number of samples in
+// view that can claim there.  Null: segments of one common capacity.
+struct SegTable {
+    const int2 *tab;
+};
+
+// Where claim number `pos` of segment i0 lies in the pair array, or -1 if the segment (or the array) is full
+// (compared as unsigned: counters that were not prepared for this problem may hold anything, and a negative
+// position must not become an address).
+__device__ __forceinline__ int fixed_position(const SegTable &segs, int pair_cap, int i0, int pos) {
+    if (segs.tab != nullptr) {
+        const int2 seg = segs.tab[i0];
+        const int at = seg.x + pos;
+        return ((unsigned)pos < (unsigned)seg.y && (unsigned)at < (unsigned)pair_cap) ? at : -1;
+    }
+    return (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
+}
 
 // Position of a kept sample's pair in the list of its first corner texel: one returning integer atomic
 // on the counter the sample's cell selects among the texel's replicas.  -1: the list is full (compared
 // as unsigned: counters that were not prepared for this problem may hold anything, and a negative
 // position must not become an address).
 __device__ __forceinline__ int claim_pair(const int *__restrict__ chunk_prefix, int *__restrict__ cursor, int pair_cap,
-                                          int texel, int cellxy) {
+                                          int texel, int cellxy, const SegTable &segs) {
     const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
     if (chunk_prefix != nullptr) {
         // counted segments: cursor holds each segment's start within its scan chunk
@@ -112,10 +131,9 @@ __device__ __forceinline__ int claim_pair(const int *__restrict__ chunk_prefix, 
         const int pos = atomicAdd(cursor + i0, 1) + chunk_prefix[i0 >> kScanChunkBits];
         return (unsigned)pos < (unsigned)pair_cap ? pos : -1;
     }
-    // fixed segments of pair_cap pairs per (texel, replica): cursor counts from zero
+    // fixed segments per (texel, replica), of pair_cap pairs each or sized by the geometry: cursor counts from zero
     const int i0 = texel * kFixedReplicas + (rep & (kFixedReplicas - 1));
-    const int pos = atomicAdd(cursor + i0, 1);
-    return (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
+    return fixed_position(segs, pair_cap, i0, atomicAdd(cursor + i0, 1));      // (the table entry travels with the atomic)
 }
 
 // Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
@@ -248,8 +266,10 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
                                                 int lane, int c_lo, int c_hi,
                                                 const int *__restrict__ chunk_prefix = nullptr,
                                                 int *__restrict__ cursor = nullptr, int pair_cap = 0,
-                                                float4 *__restrict__ store = nullptr) {
+                                                float4 *__restrict__ store = nullptr,
+                                                const SegTable segs = SegTable{nullptr}) {
     constexpr bool FILLING = MODE == kModeFill || MODE == kModeFillRuns;   // the latter claims per run
+    constexpr bool COUNTING = MODE == kModeCount || MODE == kModeCountView;
     constexpr bool BACKWARD = MODE == kModeScatter || FILLING;
     constexpr bool STORING = MODE == kModeForwardStore;      // `store`: the slot of the batch's first cell
     if (lane < k.slots_a) L.cnt[lane] = 0;
@@ -285,8 +305,8 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
             const int t10 = (rowbase + g.v0) * k.W + g.u1;
             const int t11 = (rowbase + g.v1) * k.W + g.u1;
             DepthEval e;
-            if (MODE == kModeCache) {
-                e.keep = true;       // every sample in view is listed; the depth model comes later
+            if (MODE == kModeCache || MODE == kModeCountView) {
+                e.keep = true;       // every sample in view is listed / counted; the depth model comes later
                 e.wgt = e.a = e.b = 0.0f;
                 e.k0 = e.k1 = 0;
             } else {
@@ -320,7 +340,7 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
         // after the other, and a 400 x 400 x 12 grid on 4224 texels spent half of the cell pass
         // waiting for them.  Elsewhere the shuffles cost more than the saved returning atomics.
         int run_lead = lane, run_len = 1;
-        if (MODE == kModeCount || MODE == kModeFillRuns) {
+        if (COUNTING || MODE == kModeFillRuns) {
             const int prev_keep = __shfl_up((int)keep, 1, kWave);
             const int prev_texel = __shfl_up(tx.x, 1, kWave);      // every lane takes part in the exchange
             const bool cont = keep && lane > 0 && prev_keep != 0 && prev_slot == slot && prev_texel == tx.x;
@@ -334,6 +354,12 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
         if (MODE == kModeCount) {
             if (keep && run_lead == lane)
                 atomicAdd(cursor + tx.x * kReplicas + replica_of(cellxy & 0xffff, cellxy >> 16), run_len);
+            continue;
+        }
+        if (MODE == kModeCountView) {
+            // the samples in view per fixed segment: what a segment sized by the geometry has to hold
+            if (keep && run_lead == lane)
+                atomicAdd(cursor + tx.x * kFixedReplicas + (replica_of(cellxy & 0xffff, cellxy >> 16) & (kFixedReplicas - 1)), run_len);
             continue;
         }
         // candidates are in sample order, so the lanes of one slot are contiguous: [lo, hi)
@@ -363,7 +389,7 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
             dst[1] = w2;
         }
         if (MODE == kModeFill && keep)
-            reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = claim_pair(chunk_prefix, cursor, pair_cap, tx.x, cellxy);
+            reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = claim_pair(chunk_prefix, cursor, pair_cap, tx.x, cellxy, segs);
         if (MODE == kModeFillRuns) {
             // the same, but the run's first lane claims for the whole run (same cell and texel: same
             // counter) and hands the positions out; every lane takes part in the exchange
@@ -378,7 +404,7 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
                     pos += chunk_prefix[i0 >> kScanChunkBits];
                     pos = (unsigned)pos < (unsigned)pair_cap ? pos : -1;
                 } else {
-                    pos = (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
+                    pos = fixed_position(segs, pair_cap, i0, pos);
                 }
                 reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
             }
@@ -401,7 +427,7 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
 __device__ __forceinline__ void phase_a_stored(const KParams &k, const WaveLds &L, const float *__restrict__ count,
                                                const float4 *__restrict__ store, int b, int q0, int lane,
                                                const int *__restrict__ chunk_prefix, int *__restrict__ cursor,
-                                               int pair_cap) {
+                                               int pair_cap, const SegTable &segs) {
     int mine_n = 0, mine_xy = 0;
     if (lane < k.slots_a) {
         int ix = 0, iy = 0;
@@ -439,7 +465,7 @@ __device__ __forceinline__ void phase_a_stored(const KParams &k, const WaveLds &
                 geo = make_float4(0.f, 0.f, __int_as_float(0), 0.f);
                 dw = make_float4(0.f, 0.f, 0.f, __int_as_float(1 << 16));
             }
-            geo.w = __int_as_float(claim_pair(chunk_prefix, cursor, pair_cap, __float_as_int(geo.z) >> 2, cellxy));
+            geo.w = __int_as_float(claim_pair(chunk_prefix, cursor, pair_cap, __float_as_int(geo.z) >> 2, cellxy, segs));
             L.lst[2 * j] = geo;
             L.lst[2 * j + 1] = dw;
         }

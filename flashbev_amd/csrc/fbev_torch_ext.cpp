@@ -263,7 +263,7 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                             float depth_min, float depth_step, int reduction, int backward_mode,
                             int64_t pair_capacity, std::optional<at::Tensor> cell_count, bool accumulate,
                             std::optional<at::Tensor> workspace, std::optional<at::Tensor> sample_store,
-                            std::optional<std::vector<double>> voxel_size) {
+                            std::optional<std::vector<double>> voxel_size, int workspace_layout) {
     fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
                               depth_distribution, epsilon, depth_weight_threshold, depth_min, depth_step, reduction);
     auto roi = host_floats(roi_range, 6, "roi_range");
@@ -367,11 +367,19 @@ void flash_bevpool_backward(const at::Tensor &out_grad, const at::Tensor &depth_
                     "flashbevpool_ext: a persistent workspace goes with backward_mode 0 (auto) or 2 (gather)");
         check_dev(*workspace, depth_params, "workspace");
         TORCH_CHECK(workspace->scalar_type() == at::kByte, "flashbevpool_ext: workspace must be a uint8 tensor");
+        TORCH_CHECK(workspace_layout == 1 || workspace_layout == 2,
+                    "flashbevpool_ext: workspace_layout must be 1 (segments of one capacity) or 2 (sized by the geometry)");
         if (store != nullptr)
             raise_on(fbev_backward_gather_stored(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
                                                  projection_matrices.data_ptr<float>(), stored_count, store, store_bytes, dd, df,
-                                                 accumulate ? 1 : 0, workspace->data_ptr(), (size_t)workspace->numel(), 1, st),
+                                                 accumulate ? 1 : 0, workspace->data_ptr(), (size_t)workspace->numel(),
+                                                 workspace_layout, st),
                      "fbev_backward_gather_stored");
+        else if (workspace_layout == 2)
+            raise_on(fbev_backward_gather_sized(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(), image_feats.data_ptr(),
+                                                projection_matrices.data_ptr<float>(), dd, df, accumulate ? 1 : 0,
+                                                workspace->data_ptr(), (size_t)workspace->numel(), st),
+                     "fbev_backward_gather_sized");
         else
             raise_on(fbev_backward_gather_persistent(&p, out_grad.data_ptr<float>(), depth_params.data_ptr(),
                                                      image_feats.data_ptr(), projection_matrices.data_ptr<float>(), dd, df,
@@ -404,6 +412,33 @@ int64_t backward_workspace_bytes(const at::Tensor &depth_params, const at::Tenso
     const uint64_t texels = (uint64_t)p.batch * p.num_cams * p.feat_h * p.feat_w;
     if (max_pairs == 0 || max_pairs >= (1ull << 31) || texels * 32 >= (1ull << 31)) return 0;
     return (int64_t)fbev_backward_persistent_workspace_bytes(&p);
+}
+
+// A persistent workspace whose segments are sized by the geometry (fbev_backward_workspace_init_sized): counted for
+// these matrices, this grid, region of interest, image size and epsilon; one device-to-host copy (the number of
+// samples in view) decides its size.  For flash_bevpool_backward(..., workspace_layout=2).
+at::Tensor prepare_sized_backward_workspace(const at::Tensor &depth_params, const at::Tensor &image_feats,
+                                            const at::Tensor &projection_matrices, const at::Tensor &feature_size,
+                                            const at::Tensor &image_size, const at::Tensor &grid_size,
+                                            int depth_distribution, std::vector<double> voxel_min,
+                                            std::vector<double> voxel_size, float epsilon) {
+    fbev_problem p = describe(depth_params, image_feats, projection_matrices, feature_size, image_size, grid_size,
+                              depth_distribution, epsilon, 0.0f, 1.0f, 1.0f, 0);
+    TORCH_CHECK(voxel_min.size() == 3 && voxel_size.size() == 3, "flashbevpool_ext: voxel_min and voxel_size need 3 entries each");
+    for (int a = 0; a < 3; ++a) { p.voxel_min[a] = voxel_min[a]; p.voxel_size[a] = voxel_size[a]; }
+    const size_t head = fbev_backward_sized_workspace_bytes(&p, 0), at_total = fbev_backward_sized_total_offset(&p);
+    TORCH_CHECK(head > 0 && at_total + sizeof(int32_t) <= head, "flashbevpool_ext: no sized workspace for this problem");
+    auto bytes_on = at::TensorOptions().device(depth_params.device()).dtype(at::kByte);
+    at::Tensor tables = at::empty({(int64_t)head}, bytes_on);
+    DeviceScope scope(depth_params.get_device());
+    hipStream_t st = c10::hip::getCurrentHIPStream(depth_params.get_device()).stream();
+    raise_on(fbev_backward_workspace_init_sized(&p, projection_matrices.data_ptr<float>(), tables.data_ptr(), head, st),
+             "fbev_backward_workspace_init_sized");
+    const int64_t total = tables.narrow(0, (int64_t)at_total, 4).view(at::kInt).item<int32_t>();
+    TORCH_CHECK(total >= 0, "flashbevpool_ext: sized workspace: negative sample count");
+    at::Tensor ws = at::empty({(int64_t)fbev_backward_sized_workspace_bytes(&p, (uint64_t)total)}, bytes_on);
+    ws.narrow(0, 0, (int64_t)head).copy_(tables);      // what lies in front of the pairs does not depend on their number
+    return ws;
 }
 
 at::Tensor prepare_backward_workspace(const at::Tensor &depth_params, const at::Tensor &image_feats,
@@ -554,11 +589,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("depth_min") = 1.0f, py::arg("depth_step") = 1.0f, py::arg("reduction") = 0,
           py::arg("backward_mode") = 0, py::arg("pair_capacity") = -1, py::arg("cell_count") = py::none(),
           py::arg("accumulate") = true, py::arg("workspace") = py::none(), py::arg("sample_store") = py::none(),
-          py::arg("voxel_size") = py::none());
+          py::arg("voxel_size") = py::none(), py::arg("workspace_layout") = 1);
     m.def("backward_workspace_bytes", &backward_workspace_bytes,
           "bytes of a persistent inverse-map workspace (0 when the problem is beyond the inverse map)");
     m.def("prepare_backward_workspace", &prepare_backward_workspace,
           "a persistent inverse-map workspace, allocated and prepared on the current stream");
+    m.def("prepare_sized_backward_workspace", &prepare_sized_backward_workspace,
+          "a persistent inverse-map workspace with segments sized by the geometry, prepared on the current stream",
+          py::arg("depth_params"), py::arg("image_feats"), py::arg("projection_matrices"), py::arg("feature_size"),
+          py::arg("image_size"), py::arg("grid_size"), py::arg("depth_distribution"), py::arg("voxel_min"),
+          py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);
     m.def("sample_geometry", &sample_geometry, "per-sample validity mask and corner indices (parity hook)",
           py::arg("projection_matrices"), py::arg("feat_h"), py::arg("feat_w"), py::arg("image_h"), py::arg("image_w"),
           py::arg("grid_size"), py::arg("voxel_min"), py::arg("voxel_size"), py::arg("epsilon") = 1e-6f);

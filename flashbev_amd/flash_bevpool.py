@@ -86,30 +86,98 @@ def _stream_id(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+_FIXED, _SIZED = 1, 2          # the extension's workspace_layout values
+# "auto" sizes the segments by the geometry where room for every sample would take more than this
+_SIZED_FROM_BYTES = 64 * 2 ** 20
+
+
+class _Workspace:
+    """A cache entry: the tensor, its layout, and for segments sized by the geometry what they were counted for
+    and how often in a row a call came with another geometry."""
+    __slots__ = ("tensor", "layout", "geometry", "misses")
+
+    def __init__(self, tensor, layout, geometry=None):
+        self.tensor, self.layout, self.geometry, self.misses = tensor, layout, geometry, 0
+
+
+def _workspace_layout() -> str:
+    name = os.environ.get("FLASHBEV_WORKSPACE_LAYOUT", "auto").lower()
+    if name not in ("auto", "fixed", "sized"):
+        raise ValueError(f"FLASHBEV_WORKSPACE_LAYOUT must be auto, fixed or sized, got {name!r}")
+    return name
+
+
 def _persistent_workspace(ext, depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
-                          depth_distribution):
+                          depth_distribution, geometry=None):
+    """(key, workspace tensor, layout) for this call, or (None, None, 0) when it takes a per-call workspace.
+
+    Two layouts.  Segments of one common capacity hold room for every sample (32 bytes each: 1.0 GB at
+    8 x 200 x 200 x 16 cells x 6 cameras) and serve any matrices.  Segments sized by the geometry hold room for the
+    samples in view only (a fifth of that), counted once for the matrices, sizes and region they are used with
+    (``geometry``: the matrices tensor's address and version, and the host-side values); a call with another
+    geometry prepares the workspace again (one pass over the samples and one device-to-host copy), and when that
+    happens twice in a row -- matrices that change from step to step, as under augmentation -- the shape goes
+    over to the common capacity for good.  FLASHBEV_WORKSPACE_LAYOUT = auto (sized from 64 MB on), fixed, sized."""
     keep = int(os.environ.get("FLASHBEV_WORKSPACES", "4"))
     if keep <= 0 or _capturing():
-        return None, None
+        return None, None, 0
     key = (image_feats.device.index, _stream_id(image_feats.device),
            tuple(image_feats.shape), depth_params.shape[-1], tuple(grid_t.tolist()), int(depth_distribution))
-    ws = _workspaces.get(key)
-    if ws is None:
-        nbytes = ext.backward_workspace_bytes(depth_params, image_feats, projection_matrices, fs_host, image_t,
-                                              grid_t, int(depth_distribution))
-        limit_mb = float(os.environ.get("FLASHBEV_WORKSPACE_MB", "16384"))
-        total_mb = float(os.environ.get("FLASHBEV_WORKSPACE_CACHE_MB", "4096"))
-        if nbytes == 0 or nbytes > min(limit_mb, total_mb) * 2 ** 20:
-            return None, None
-        ws = ext.prepare_backward_workspace(depth_params, image_feats, projection_matrices, fs_host, image_t,
-                                            grid_t, int(depth_distribution))
-        _workspaces[key] = ws
-        # the least recently used go first, until both the count and the total size fit
-        while len(_workspaces) > keep or sum(t.numel() for t in _workspaces.values()) > total_mb * 2 ** 20:
-            _workspaces.popitem(last=False)
+    limit = min(float(os.environ.get("FLASHBEV_WORKSPACE_MB", "16384")),
+                float(os.environ.get("FLASHBEV_WORKSPACE_CACHE_MB", "4096"))) * 2 ** 20
+    entry = _workspaces.get(key)
+
+    def fixed_bytes():
+        return ext.backward_workspace_bytes(depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
+                                            int(depth_distribution))
+
+    def make(layout):
+        if layout == _SIZED:
+            vmin, vsize, eps = geometry[2], geometry[3], geometry[4]
+            t = ext.prepare_sized_backward_workspace(depth_params, image_feats, projection_matrices, fs_host, image_t,
+                                                     grid_t, int(depth_distribution), list(vmin), list(vsize), eps)
+            return _Workspace(t, _SIZED, geometry) if t.numel() <= limit else None
+        t = ext.prepare_backward_workspace(depth_params, image_feats, projection_matrices, fs_host, image_t, grid_t,
+                                           int(depth_distribution))
+        return _Workspace(t, _FIXED)
+
+    if entry is None:
+        worst = fixed_bytes()
+        if worst == 0:
+            return None, None, 0
+        want = _workspace_layout()
+        sized = geometry is not None and (want == "sized" or (want == "auto" and worst > _SIZED_FROM_BYTES))
+        if not sized and worst > limit:
+            return None, None, 0
+        entry = make(_SIZED if sized else _FIXED)
+        if entry is None:
+            return None, None, 0
+    elif entry.layout == _SIZED and entry.geometry != geometry:
+        entry.misses += 1
+        worst = fixed_bytes()
+        if entry.misses >= 2 and _workspace_layout() != "sized":
+            # the geometry changes from call to call: room for every sample serves them all
+            if worst > limit:
+                _workspaces.pop(key, None)
+                return None, None, 0
+            entry = make(_FIXED)
+        else:
+            misses = entry.misses
+            entry = make(_SIZED)
+            if entry is None:
+                _workspaces.pop(key, None)
+                return None, None, 0
+            entry.misses = misses
     else:
-        _workspaces.move_to_end(key)
-    return key, ws
+        entry.misses = 0
+    _workspaces[key] = entry
+    _workspaces.move_to_end(key)
+    # the least recently used go first, until both the count and the total size fit
+    while len(_workspaces) > keep or sum(e.tensor.numel() for e in _workspaces.values()) > limit:
+        if len(_workspaces) == 1:
+            break
+        _workspaces.popitem(last=False)
+    return key, entry.tensor, entry.layout
 
 
 def _sample_store_limit() -> int:
@@ -314,6 +382,7 @@ class FlashBEVPool(torch.autograd.Function):
             ctx.counts = counts
             ctx.sample_store = store
             ctx.voxel_size = list(vsize)          # the backward takes the cell size the forward was given
+            ctx.voxel_min = list(vmin)
             ctx.pair_capacity = _pair_capacity(B, N, grid)
             ctx.host = (fs_host, image_t, roi_t, grid_t)
             ctx.total_threads = out.numel()
@@ -340,16 +409,19 @@ class FlashBEVPool(torch.autograd.Function):
                                  device=image_feats.device) if need_feats else None
         if need_depth or need_feats:
             key = ws = None
+            layout = _FIXED
             if mode in (0, 2) and ctx.pair_capacity < 0:
-                key, ws = _persistent_workspace(ext, depth_params, image_feats, projection_matrices, fs_host,
-                                                image_t, grid_t, ctx.depth_distribution)
+                geometry = (projection_matrices.data_ptr(), projection_matrices._version, tuple(ctx.voxel_min),
+                            tuple(ctx.voxel_size), ctx.epsilon, tuple(image_t.tolist()))
+                key, ws, layout = _persistent_workspace(ext, depth_params, image_feats, projection_matrices, fs_host,
+                                                        image_t, grid_t, ctx.depth_distribution, geometry)
             try:
                 ext.flash_bevpool_backward(
                     out_grad.contiguous().float(), depth_params, image_feats, projection_matrices,
                     fs_host, image_t, roi_t, grid_t, depth_params_grad, image_feats_grad,
                     ctx.total_threads, ctx.depth_distribution, ctx.epsilon, ctx.depth_weight_threshold,
                     ctx.depth_range[0], ctx.depth_range[1], ctx.reduction, mode, ctx.pair_capacity, ctx.counts, False,
-                    ws, ctx.sample_store if mode in (0, 2) else None, ctx.voxel_size)
+                    ws, ctx.sample_store if mode in (0, 2) else None, ctx.voxel_size, layout or _FIXED)
             except Exception:
                 _workspaces.pop(key, None)       # a failed call leaves a persistent workspace undefined
                 raise

@@ -179,14 +179,46 @@ int fbev_backward_gather_persistent(const fbev_problem *p, const float *grad_out
                                     int accumulate, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * A persistent workspace whose segments are sized by the geometry.  fbev_backward_gather_persistent keeps room for
+ * every (cell, camera, height) sample, in segments of one common capacity: 32 bytes x B x gy x gx x N x gz
+ * (0.98 GB for 8 x 200 x 200 cells x 6 cameras x 16 bins) of which a call fills under a tenth, because only one
+ * sample in six is in view and the texels on the horizon collect ten times the average.  Which samples are in view
+ * depends on the projection matrices and the grid only, so a workspace prepared for one set of matrices can give
+ * each (texel, replica) segment exactly the room its samples in view need:
+ *   fbev_backward_workspace_init_sized   zero-fills everything but the pairs, counts the samples in view per
+ *       segment and prefix-sums the counts (one pass over the samples, once); `workspace` needs at least
+ *       fbev_backward_sized_workspace_bytes(p, 0) bytes for that.  The total number of pairs the segments hold is
+ *       then the int32 at byte offset fbev_backward_sized_total_offset(p) of the workspace: the caller reads it
+ *       (the one device-to-host copy of this interface), allocates fbev_backward_sized_workspace_bytes(p, total)
+ *       bytes and either prepares that memory the same way or copies the first
+ *       fbev_backward_sized_workspace_bytes(p, 0) bytes over: what lies in front of the pairs does not depend on
+ *       their number.
+ *   fbev_backward_gather_sized   is fbev_backward_gather_persistent on such a workspace: two launches, same
+ *       results, same contract (one call at a time, prepared again after a failed call or a change of batch,
+ *       cameras, feature-map size, channels or depth bins), and in addition: prepared again whenever proj, the
+ *       grid, the image size, the region of interest or epsilon change.  Nothing breaks if they change without
+ *       that: a sample that finds its segment full (or a pair array shorter than the total) is added with atomics,
+ *       as everywhere; it only costs time.
+ * No counterpart in the reference, whose backward keeps no workspace (flash_bevpool_cuda.cu:867-937).
+ */
+size_t fbev_backward_sized_workspace_bytes(const fbev_problem *p, uint64_t pair_capacity);
+size_t fbev_backward_sized_total_offset(const fbev_problem *p);
+int fbev_backward_workspace_init_sized(const fbev_problem *p, const float *proj, void *workspace, size_t workspace_bytes,
+                                       void *stream);
+int fbev_backward_gather_sized(const fbev_problem *p, const float *grad_out, const void *depth, const void *feats,
+                               const float *proj, float *d_depth, float *d_feats, int accumulate, void *workspace,
+                               size_t workspace_bytes, void *stream);
+
+/*
  * Forward and backward of one differentiated call sharing the sample evaluation.  fbev_forward_store is
  * fbev_forward (same `out`, same `count_out`, which is required here) that also leaves, for every kept
  * sample, a 32-byte record (bilinear fractions, first corner texel with the two clamp flags, depth weight
  * and its two derivative terms, depth bins) in `store`: caller-owned device memory of
  * fbev_sample_store_bytes(p) bytes, 16-byte aligned, one slot of N * grid_z records per BEV cell, i.e.
  * B * ceil(gx/8) * ceil(gy/8) * 64 * N * grid_z * 32 bytes (0: outside the limits, B*N*H*W >= 2^29); only the
- * records of kept samples are written.  fbev_backward_gather_stored is fbev_backward_gather (persistent == 0)
- * or fbev_backward_gather_persistent (persistent != 0, `workspace` prepared as described there) whose cell
+ * records of kept samples are written.  fbev_backward_gather_stored is fbev_backward_gather (persistent == 0),
+ * fbev_backward_gather_persistent (persistent == 1) or fbev_backward_gather_sized (persistent == 2), with
+ * `workspace` prepared as described there, whose cell
  * pass copies those records instead of projecting and weighting every sample again; `cell_count` and `store`
  * are what fbev_forward_store wrote for the same p, depth, feats and proj.  Same gradients as
  * fbev_backward_gather, to rounding.  It pays where a call is bound by latency rather than throughput (small

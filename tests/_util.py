@@ -101,21 +101,42 @@ def capi_forward_cached(x, w, dist, cache, thr=1e-6, eps=1e-6, reduction=capi.FB
     return (out, cnt) if with_count else out
 
 
+def sized_workspace(p, proj, pair_capacity=None):
+    """A persistent workspace with segments sized for the matrices `proj`: the tables first, then, once the number
+    of samples in view has been read back, the whole of it.  Returns (tensor, pairs in view)."""
+    dev = proj.device
+    st = torch.cuda.current_stream().cuda_stream
+    head = capi.backward_sized_workspace_bytes(p, 0)
+    tables = torch.empty(head, dtype=torch.uint8, device=dev).fill_(0x5A)
+    capi.check(capi.backward_workspace_init_sized(p, proj.data_ptr(), tables.data_ptr(), head, st),
+               "fbev_backward_workspace_init_sized")
+    at = capi.backward_sized_total_offset(p)
+    total = int(tables[at:at + 4].view(torch.int32).item())
+    nbytes = capi.backward_sized_workspace_bytes(p, total if pair_capacity is None else pair_capacity)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(0x5A)
+    ws[:head].copy_(tables)
+    return ws, total
+
+
 def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEAN, want=(True, True),
-                  mode="scatter", pair_capacity=None):
+                  mode="scatter", pair_capacity=None, sized_for=None):
     """Backward through the C ABI.  mode "scatter" = fbev_backward, "gather" = fbev_backward_gather
     with a workspace for `pair_capacity` pairs (default: the worst case, which selects fixed
     per-texel segments; "gather_counted" defaults to half of that, the exactly packed layout), "columns" =
     fbev_backward_columns overwriting NaN-filled buffers with recounted cell counts, "persistent" =
     fbev_backward_gather_persistent on a workspace prepared once (three calls in a row, the last one returned),
     "columns_acc" = the same accumulating into zero-filled buffers with the forward's counts,
+    "sized" = fbev_backward_gather_sized on a workspace whose segments fbev_backward_workspace_init_sized sized for
+    `sized_for` (default: these matrices; `pair_capacity` shortens its pair array), three calls in a row,
+    "stored_sized" = the same through the forward's sample store,
     "stored" / "stored_persistent" = fbev_forward_store (whose output and counts must equal fbev_forward's bit
     for bit) followed by fbev_backward_gather_stored on a per-call / a persistent workspace (twice in a row on
     the persistent one)."""
     p = problem_for(x, w, dist, thr, eps, reduction)
     dev = x["image_feats"].device
     overwrite = mode in ("columns", "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite",
-                         "persistent_overwrite", "stored_overwrite", "stored_persistent_overwrite")
+                         "persistent_overwrite", "stored_overwrite", "stored_persistent_overwrite", "sized_overwrite",
+                         "stored_sized_overwrite")
     fill = float("nan") if overwrite else 0.0
     dd = torch.full(x["depth_params"].shape, fill, dtype=torch.float32, device=dev) if want[0] else None
     df = torch.full(x["image_feats"].shape, fill, dtype=torch.float32, device=dev) if want[1] else None
@@ -138,8 +159,19 @@ def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEA
             _, cnt = capi_forward(x, w, dist, thr, eps, reduction, with_count=True)
             capi.check(capi.backward_columns(p, *args, cnt.data_ptr(), ddp, dfp, True, None, 0, st),
                        "fbev_backward_columns")
+    elif mode in ("sized", "sized_overwrite"):
+        ws, _ = sized_workspace(p, x["projection_matrices"] if sized_for is None else sized_for, pair_capacity)
+        for call in range(3):
+            if dd is not None:
+                dd.fill_(fill)
+            if df is not None:
+                df.fill_(fill)
+            capi.check(capi.backward_gather_sized(p, x["grad_out"].data_ptr(), x["depth_params"].data_ptr(),
+                                                  x["image_feats"].data_ptr(), x["projection_matrices"].data_ptr(),
+                                                  ddp, dfp, ws.data_ptr(), ws.numel(), st, accumulate=not overwrite),
+                       "fbev_backward_gather_sized")
     elif mode.startswith("stored"):
-        persistent = "persistent" in mode
+        persistent = 2 if "sized" in mode else (1 if "persistent" in mode else 0)
         out, cnt = capi_forward(x, w, dist, thr, eps, reduction, with_count=True)
         sbytes = capi.sample_store_bytes(p)
         assert sbytes > 0
@@ -151,7 +183,10 @@ def capi_backward(x, w, dist, thr=1e-6, eps=1e-6, reduction=capi.FBEV_REDUCE_MEA
                                       store.data_ptr(), sbytes, st), "fbev_forward_store")
         torch.cuda.synchronize()
         assert torch.equal(out2, out) and torch.equal(cnt2, cnt), "fbev_forward_store differs from fbev_forward"
-        if persistent:
+        if persistent == 2:
+            ws, _ = sized_workspace(p, x["projection_matrices"] if sized_for is None else sized_for, pair_capacity)
+            nbytes = ws.numel()
+        elif persistent:
             nbytes = capi.backward_persistent_workspace_bytes(p)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(0x5A)
             capi.check(capi.backward_workspace_init(p, ws.data_ptr(), nbytes, st), "fbev_backward_workspace_init")

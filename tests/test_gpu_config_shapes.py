@@ -80,7 +80,8 @@ BACKWARD_CASES = [("cfg4_hires", 1, "gather"), ("cfg4_hires", 2, "gather"), ("cf
                   ("cfg2_surround", 1, "persistent_overwrite"), ("cfg3_zsweep", 1, "persistent"),
                   ("cfg4_hires", 2, "persistent_overwrite"), ("cfg5_train", 1, "persistent_overwrite"),
                   ("cfg3_zsweep", 2, "stored_persistent_overwrite"), ("cfg4_hires", 1, "stored"),
-                  ("cfg5_train", 0, "stored_persistent_overwrite")]
+                  ("cfg5_train", 0, "stored_persistent_overwrite"), ("cfg3_zsweep", 1, "sized"),
+                  ("cfg4_hires", 2, "sized_overwrite"), ("cfg5_train", 1, "sized_overwrite")]
 
 
 @pytest.mark.parametrize("name,dist,mode", BACKWARD_CASES)
@@ -95,6 +96,30 @@ def test_backward_against_the_oracle_at_the_configurations_own_shape(name, dist,
     for got, ref, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
         bad, maxabs, ratio = U.violations(got.cpu().numpy(), ref)
         assert bad == 0, (what, bad, maxabs, ratio)
+
+
+def test_sized_segments_hold_every_sample_in_view_and_a_fifth_of_the_memory():
+    """At the training size: the segments sized by the geometry hold exactly the oracle's number of samples in view
+    (so no call on these matrices ever finds one full, whatever the depth tensor and the threshold), in under
+    300 MB where room for every sample takes a gigabyte; and a workspace sized for the first batch element's
+    matrices alone (every batch element has its own jitter) still gives the right gradients: what finds no room
+    is added with atomics."""
+    w = workload("cfg5_train")
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=True)
+    p = U.problem_for(x, w, 1, thr=0.0)
+    ws, total = U.sized_workspace(p, x["projection_matrices"])
+    geo = c_oracle.geometry(x["projection_matrices"].cpu().numpy(), w.feat_hw, w.image_hw, w.roi_range, w.grid_size)
+    assert total == int(geo["mask"].sum())
+    assert ws.numel() < 300e6 and capi.backward_persistent_workspace_bytes(p) > 1000e6
+    del ws, geo
+    # threshold 0 keeps every sample in view: every segment is filled to the brim, none overflows
+    dd, df = U.capi_backward(x, w, 1, thr=0.0, mode="sized_overwrite")
+    want_dd, want_df = U.oracle_backward(x, w, 1, thr=0.0)
+    assert U.violations(df.cpu().numpy(), want_df)[0] == 0 and U.violations(dd.cpu().numpy(), want_dd)[0] == 0
+    same = x["projection_matrices"][:1].expand_as(x["projection_matrices"]).contiguous()
+    dd, df = U.capi_backward(x, w, 1, thr=0.0, mode="sized_overwrite", sized_for=same)
+    assert U.violations(df.cpu().numpy(), want_df, rtol=3e-4, atol=3e-5)[0] == 0
+    assert U.violations(dd.cpu().numpy(), want_dd, rtol=3e-4, atol=3e-5)[0] == 0
 
 
 CACHED_CASES = [("cfg1_tiny", None, 0), ("cfg2_surround", None, 1), ("cfg2_surround", None, 2), ("cfg3_zsweep", 12, 1),

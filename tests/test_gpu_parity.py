@@ -60,7 +60,8 @@ def test_forward_matches_c_oracle(name, dist, thr):
 @pytest.mark.parametrize("mode", ["scatter", "gather", "gather_counted", "columns", "columns_acc",
                                   "scatter_overwrite", "gather_overwrite", "gather_counted_overwrite",
                                   "persistent", "persistent_overwrite", "stored", "stored_overwrite",
-                                  "stored_persistent", "stored_persistent_overwrite"])
+                                  "stored_persistent", "stored_persistent_overwrite", "sized", "sized_overwrite",
+                                  "stored_sized_overwrite"])
 def test_backward_matches_c_oracle(name, dist, mode):
     w, x = _inputs(name, dist)
     dd, df = U.capi_backward(x, w, dist, mode=mode)
@@ -89,6 +90,24 @@ def test_backward_from_the_sample_store_with_short_workspace(capacity):
     want_dd, want_df = U.oracle_backward(x, w, 2)
     assert U.violations(df.cpu().numpy(), want_df)[0] == 0
     assert U.violations(dd.cpu().numpy(), want_dd)[0] == 0
+
+
+@pytest.mark.parametrize("dist", [1, 2])
+def test_segments_sized_for_another_geometry_or_a_short_pair_array_fall_back_to_atomics(dist):
+    """A workspace whose segments were sized for other matrices (the cameras in another order: the samples in view
+    land on other texels), and one whose pair array holds a third of the samples in view: whatever finds no room is
+    added with atomics, so the gradients are the oracle's all the same.  (Sums of many fp32 terms in an order
+    the atomics do not fix: three times the usual tolerance, as for the other overflow cases.)"""
+    w, x = _inputs("cfg2_surround", dist)
+    want_dd, want_df = U.oracle_backward(x, w, dist)
+    p = U.problem_for(x, w, dist)
+    other = x["projection_matrices"].flip(1).roll(1, 1).contiguous()
+    _, total = U.sized_workspace(p, x["projection_matrices"])
+    for kw in (dict(sized_for=other), dict(pair_capacity=total // 3), dict(pair_capacity=0)):
+        for mode in ("sized", "sized_overwrite", "stored_sized_overwrite"):
+            dd, df = U.capi_backward(x, w, dist, mode=mode, **kw)
+            assert U.violations(df.cpu().numpy(), want_df, rtol=3e-4, atol=3e-5)[0] == 0, (kw.keys(), mode)
+            assert U.violations(dd.cpu().numpy(), want_dd, rtol=3e-4, atol=3e-5)[0] == 0, (kw.keys(), mode)
 
 
 def test_a_foreign_sample_store_gives_no_access_out_of_bounds():

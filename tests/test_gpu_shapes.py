@@ -314,6 +314,9 @@ def test_fixed_segments_overflow_falls_back_to_atomics(dist):
     # fix: three times the usual tolerance (observed: up to 1.01 times the usual one)
     check_all(w, x, dist, thr=0.0, modes=("gather", "gather_overwrite", "gather_counted", "persistent",
                                           "persistent_overwrite"), bwd_tol=(3e-4, 3e-5))
+    # segments sized by the geometry hold these texels' thousands of samples: nothing overflows (the sums are as
+    # long and their order as free, hence the same tolerance)
+    check_all(w, x, dist, thr=0.0, modes=("sized", "sized_overwrite"), bwd_tol=(3e-4, 3e-5))
 
 
 def test_the_reference_calibration_fixture():

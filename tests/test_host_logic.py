@@ -176,6 +176,10 @@ class FakeExt:
         self.prepared = getattr(self, "prepared", 0) + 1
         return torch.zeros(4096, dtype=torch.uint8)
 
+    def prepare_sized_backward_workspace(self, *a):
+        self.prepared_sized = getattr(self, "prepared_sized", 0) + 1
+        return torch.zeros(2048, dtype=torch.uint8)
+
 
 @pytest.fixture
 def fake_ext(monkeypatch):
@@ -187,6 +191,43 @@ def fake_ext(monkeypatch):
     # the operator insists on a GPU tensor; let CPU tensors pass for this host-logic test
     monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
     return ext
+
+
+def test_workspace_layout_follows_the_size_and_the_geometry(fake_ext, monkeypatch):
+    """Where room for every sample would take more than 64 MB the cached workspace gets segments sized by the
+    geometry: kept while the matrices tensor stays the same (same storage, same version), prepared again when it
+    changes, and replaced by the common-capacity layout once the geometry has changed twice in a row."""
+    w = WORKLOADS["cfg1_tiny"]
+    x = make_inputs(w, "parametric")
+    monkeypatch.setattr(fake_ext, "backward_workspace_bytes", lambda *a: 100 * 2 ** 20)
+
+    def step(proj):
+        f = x["image_feats"].clone().requires_grad_(True)
+        flash_bevpool(f, x["depth_params"], proj, x["feature_size"], x["image_size"], x["roi_range"],
+                      x["grid_size"]).sum().backward()
+        return fake_ext.bwd[-4], fake_ext.bwd[-1]            # workspace, layout
+
+    proj = x["projection_matrices"]
+    ws, layout = step(proj)
+    assert layout == 2 and ws.numel() == 2048 and fake_ext.prepared_sized == 1
+    assert step(proj)[0] is ws and fake_ext.prepared_sized == 1          # same geometry: kept
+    proj.mul_(1.0)                                                       # modified in place: another geometry
+    ws2, layout = step(proj)
+    assert layout == 2 and ws2 is not ws and fake_ext.prepared_sized == 2
+    assert step(proj)[0] is ws2                                          # settles again: the miss count starts over
+    ws3, layout = step(proj.clone())
+    assert layout == 2 and fake_ext.prepared_sized == 3
+    ws4, layout = step(proj.clone())                                     # the second change in a row
+    assert layout == 1 and ws4.numel() == 4096 and getattr(fake_ext, "prepared", 0) == 1
+    assert step(proj.clone())[0] is ws4                                  # and stays there
+    # the layout can be forced either way
+    op_module._workspaces.clear()
+    monkeypatch.setenv("FLASHBEV_WORKSPACE_LAYOUT", "fixed")
+    assert step(proj)[1] == 1
+    op_module._workspaces.clear()
+    monkeypatch.setenv("FLASHBEV_WORKSPACE_LAYOUT", "sized")
+    for _ in range(4):
+        assert step(proj.clone())[1] == 2                                # never gives up on sized segments when told so
 
 
 def test_sample_store_goes_with_small_differentiated_calls_only(fake_ext, monkeypatch):
@@ -207,13 +248,13 @@ def test_sample_store_goes_with_small_differentiated_calls_only(fake_ext, monkey
     gx, gy, gz = w.grid_size
     want = w.batch * ((gx + 7) // 8) * ((gy + 7) // 8) * 64 * w.num_cams * gz * 32
     assert store is not None and store.dtype == torch.uint8 and store.numel() == want
-    assert fake_ext.bwd[-2] is store
+    assert fake_ext.bwd[-3] is store
     assert call(False) is None
     monkeypatch.setenv("FLASHBEV_SAMPLE_STORE_MB", str((want - 1) / 2 ** 20))
-    assert call(True) is None and fake_ext.bwd[-2] is None
+    assert call(True) is None and fake_ext.bwd[-3] is None
     monkeypatch.setenv("FLASHBEV_SAMPLE_STORE_MB", "64")
     monkeypatch.setenv("FLASHBEV_BACKWARD", "columns")
-    assert call(True) is None and fake_ext.bwd[-2] is None
+    assert call(True) is None and fake_ext.bwd[-3] is None
 
 
 def test_operator_marshalling_matches_reference_order(fake_ext):
@@ -247,7 +288,7 @@ def test_persistent_workspace_is_prepared_once_per_shape_and_dropped_when_switch
         out = flash_bevpool(f, x["depth_params"], x["projection_matrices"], x["feature_size"], x["image_size"],
                             x["roi_range"], x["grid_size"] if grid is None else grid)
         out.sum().backward()
-        return fake_ext.bwd[-3]
+        return fake_ext.bwd[-4]
 
     ws = step()
     assert ws is not None and ws.dtype == torch.uint8 and fake_ext.prepared == 1
