@@ -266,15 +266,22 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coefs[q], g[q][v], acc[v]);
             }
-            for (int i = full; i < n_lead; i += wpw) {
-                const int j = i + wslot_eff;
-                if (j < n_lead) {
-                    const float2 rc = stage[j];
-                    float g[VEC];
-                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g);
+            if (full < n_lead) {
+                // the rest as one more group, its gathers in flight together: a worker past the last row takes
+                // the last row again with a coefficient of zero
+                float coefs[UNR];
+                float g[UNR][VEC];
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(rc.y, g[v], acc[v]);
+                for (int q = 0; q < UNR; ++q) {
+                    const int want = full + q * wpw + wslot_eff;
+                    const float2 rc = stage[min(want, n_lead - 1)];
+                    coefs[q] = want < n_lead ? rc.y : 0.0f;
+                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g[q]);
                 }
+#pragma unroll
+                for (int q = 0; q < UNR; ++q)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(coefs[q], g[q][v], acc[v]);
             }
             __builtin_amdgcn_wave_barrier();      // the records are read before the next chunk overwrites them
         }
