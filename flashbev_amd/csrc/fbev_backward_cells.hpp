@@ -158,12 +158,19 @@ __global__ __launch_bounds__(1024) void fbev_scan_sums_kernel(int *v, int n) {
 }
 
 // The table of segments sized by the geometry: absolute start and capacity of every segment, from the
-// capacities, their prefix sums within chunks of 4096 and the chunks' prefix sums.
+// capacities, their prefix sums within chunks of 4096 and the chunks' prefix sums; and the segments' packed
+// claim counters in their initial state, in both sets (set_stride 32-bit words apart).
 __global__ __launch_bounds__(256) void fbev_segment_table_kernel(long long n, const int *__restrict__ cap,
                                                                  const int *__restrict__ off,
-                                                                 const int *__restrict__ prefix, int2 *__restrict__ tab) {
+                                                                 const int *__restrict__ prefix, int2 *__restrict__ tab,
+                                                                 int *__restrict__ sets, long long set_stride) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) tab[i] = make_int2(prefix[i >> kScanChunkBits] + off[i], cap[i]);
+    if (i >= n) return;
+    const int start = prefix[i >> kScanChunkBits] + off[i];
+    tab[i] = make_int2(start, cap[i]);
+    const unsigned long long word = packed_counter(start, cap[i]);
+    reinterpret_cast<unsigned long long *>(sets)[i] = word;
+    reinterpret_cast<unsigned long long *>(sets + set_stride)[i] = word;
 }
 
 // Cell pass of the backward.  FILL = 0: scatter with atomics.  FILL = 1: write pairs (inverse

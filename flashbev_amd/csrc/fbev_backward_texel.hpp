@@ -82,6 +82,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     const int tu = t % k.W, tv = (t / k.W) % k.H;
     int my_lo = 0, my_len = 0;
     bool spilled = false;      // a list of this texel was full: the cell pass added the rest with atomics
+    unsigned long long own_word = 0;   // (packed counters) the initial state of the counter of an own segment
     if (lane < kTexelSegs) {
         const int e = lane;
         const int o = counted ? e : e & 3;
@@ -99,15 +100,20 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             // fixed segments of pair_cap pairs; seg_end holds how many were claimed
             const int i = q * kFixedReplicas + (e >> 2);
             my_lo = i * pair_cap;
-            int room = pair_cap;
+            int room = pair_cap, seg_cap = 0;
             if (ps.segs.tab != nullptr) {
                 // (a segment that would reach past the pair array holds what fits: the rest was added with atomics)
                 const int2 seg = ps.segs.tab[i];
                 my_lo = seg.x;
+                seg_cap = seg.y;
                 room = max(min(seg.y, pair_cap - my_lo), 0);
             }
             int claimed;
-            if (persistent) {
+            if (ps.segs.tab != nullptr) {
+                // packed counters: the low word started at kSegBias - capacity
+                const int in_first = ps.sets[2 * i], in_second = ps.sets[ps.set_stride + 2 * i];
+                claimed = (int)((unsigned)(set ? in_second : in_first) - (kSegBias - (unsigned)seg_cap));
+            } else if (persistent) {
                 const int in_first = ps.sets[i], in_second = ps.sets[ps.set_stride + i];
                 claimed = set ? in_second : in_first;
             } else {
@@ -115,12 +121,20 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             }
             spilled = claimed > room;
             my_len = max(min(claimed, room), 0);
+            if (o == 0) own_word = packed_counter(my_lo, seg_cap);
         }
     }
-    if (persistent && threadIdx.x == 0 && blockIdx.y == 0) {
-        // the counters of this texel in the set the next call claims in
-        *reinterpret_cast<int4 *>(ps.sets + (size_t)(set ^ 1) * ps.set_stride + (size_t)t * kFixedReplicas) = make_int4(0, 0, 0, 0);
-        if (blockIdx.x == 0) ps.epoch[1] = epoch + 1;
+    if (persistent && blockIdx.y == 0) {
+        // the counters of this texel in the set the next call claims in: zero, or, packed, their initial state
+        // (lists 0, 4, 8, 12 are the texel's own segments, one per replica)
+        int *next = ps.sets + (size_t)(set ^ 1) * ps.set_stride;
+        if (ps.segs.tab != nullptr) {
+            if (threadIdx.x < kTexelSegs && (threadIdx.x & 3) == 0)
+                reinterpret_cast<unsigned long long *>(next)[(size_t)t * kFixedReplicas + (threadIdx.x >> 2)] = own_word;
+        } else if (threadIdx.x == 0) {
+            *reinterpret_cast<int4 *>(next + (size_t)t * kFixedReplicas) = make_int4(0, 0, 0, 0);
+        }
+        if (blockIdx.x == 0 && threadIdx.x == 0) ps.epoch[1] = epoch + 1;
     }
     // the lists one after the other form one sequence of pairs; list e starts at my_pre of lane e
     int my_pre = my_len;

@@ -462,7 +462,8 @@ size_t ws_index_bytes(const fbev_problem *p) {
 // within scan chunks of 4096 segments, and per chunk the pairs before it, with the total behind the last chunk.
 struct PersistLayout {
     size_t sets, ovf_depth, ovf_feats, pairs;      // byte offsets
-    long long set_stride;                          // ints between the two sets
+    long long segments;                            // (texel, replica) segments = claim counters per set
+    long long set_stride;                          // ints between the two sets (sized segments: 64-bit counters)
     size_t seg_tab, seg_cap, seg_off, seg_prefix;  // byte offsets of the tables (sized segments only)
     long long seg_chunks;                          // scan chunks of the segment tables
 };
@@ -470,18 +471,19 @@ PersistLayout persist_layout(const fbev_problem *p, bool sized = false) {
     auto pad = [](size_t n) { return (n + 255) / 256 * 256; };
     const size_t texels = (size_t)texel_count(p);
     PersistLayout l;
-    l.set_stride = (long long)texels * kFixedReplicas;
+    l.segments = (long long)texels * kFixedReplicas;
+    l.set_stride = sized ? 2 * l.segments : l.segments;
     l.sets = 256;
     l.ovf_depth = l.sets + pad(2 * (size_t)l.set_stride * sizeof(int));
     l.ovf_feats = l.ovf_depth + pad(texels * p->depth_bins * sizeof(float));
     l.pairs = l.ovf_feats + pad(texels * p->channels * sizeof(float));
     l.seg_tab = l.seg_cap = l.seg_off = l.seg_prefix = 0;
-    l.seg_chunks = (l.set_stride + (1ll << kScanChunkBits) - 1) >> kScanChunkBits;
+    l.seg_chunks = (l.segments + (1ll << kScanChunkBits) - 1) >> kScanChunkBits;
     if (sized) {
         l.seg_tab = l.pairs;
-        l.seg_cap = l.seg_tab + pad((size_t)l.set_stride * sizeof(int2));
-        l.seg_off = l.seg_cap + pad((size_t)l.set_stride * sizeof(int));
-        l.seg_prefix = l.seg_off + pad((size_t)l.set_stride * sizeof(int));
+        l.seg_cap = l.seg_tab + pad((size_t)l.segments * sizeof(int2));
+        l.seg_off = l.seg_cap + pad((size_t)l.segments * sizeof(int));
+        l.seg_prefix = l.seg_off + pad((size_t)l.segments * sizeof(int));
         l.pairs = l.seg_prefix + pad((size_t)(l.seg_chunks + 1) * sizeof(int));
     }
     return l;
@@ -738,12 +740,12 @@ int workspace_init_sized_impl(const fbev_problem *p, const float *proj, void *wo
     int *seg_prefix = reinterpret_cast<int *>(base + lay.seg_prefix);
     rc = launch_count<float, true>(pl, nullptr, proj, seg_cap, st);
     if (rc != FBEV_OK) return rc;
-    if (hipMemcpyAsync(seg_off, seg_cap, (size_t)lay.set_stride * sizeof(int), hipMemcpyDeviceToDevice, st) != hipSuccess)
+    if (hipMemcpyAsync(seg_off, seg_cap, (size_t)lay.segments * sizeof(int), hipMemcpyDeviceToDevice, st) != hipSuccess)
         return FBEV_ERR_LAUNCH;
     {
         prof::Scope timer(prof::kScanChunks, st);
         hipLaunchKernelGGL(fbev_scan_chunks_kernel, dim3((unsigned)lay.seg_chunks), dim3(1024), 0, st, seg_off,
-                           lay.set_stride, seg_prefix);
+                           lay.segments, seg_prefix);
     }
     if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
     {
@@ -752,8 +754,9 @@ int workspace_init_sized_impl(const fbev_problem *p, const float *proj, void *wo
         hipLaunchKernelGGL(fbev_scan_sums_kernel, dim3(1), dim3(1024), 0, st, seg_prefix, (int)lay.seg_chunks + 1);
     }
     if (hipGetLastError() != hipSuccess) return FBEV_ERR_LAUNCH;
-    hipLaunchKernelGGL(fbev_segment_table_kernel, dim3((unsigned)((lay.set_stride + 255) / 256)), dim3(256), 0, st,
-                       lay.set_stride, seg_cap, seg_off, seg_prefix, reinterpret_cast<int2 *>(base + lay.seg_tab));
+    hipLaunchKernelGGL(fbev_segment_table_kernel, dim3((unsigned)((lay.segments + 255) / 256)), dim3(256), 0, st,
+                       lay.segments, seg_cap, seg_off, seg_prefix, reinterpret_cast<int2 *>(base + lay.seg_tab),
+                       reinterpret_cast<int *>(base + lay.sets), lay.set_stride);
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }
 

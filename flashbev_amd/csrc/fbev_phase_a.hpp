@@ -102,19 +102,30 @@ enum { kModeForward = 0, kModeScatter = 1, kModeFill = 2, kModeCount = 3, kModeF
 // Segments sized by the geometry (a persistent workspace prepared for one set of matrices): segment i =
 // (texel, replica) starts at tab[i].x in the pair array and has room for tab[i].y pairs, the number of samples in
 // view that can claim there.  Null: segments of one common capacity.
+// The claim counter of such a segment is a 64-bit word that carries the segment along, so that the one returning
+// atomic of a claim brings back all a claim needs:
+//   low word   kSegBias - capacity + claims so far: the sign bit comes on with the first claim that does not fit
+//   high word  start + capacity - kSegBias:         low + high (mod 2^32) = start + claims so far, the position
+// (fewer than 2^31 samples exist, so the low word never carries into the high one).
 struct SegTable {
     const int2 *tab;
 };
+constexpr unsigned kSegBias = 0x80000000u;
+__host__ __device__ __forceinline__ unsigned long long packed_counter(int start, int cap) {
+    return ((unsigned long long)((unsigned)start + (unsigned)cap - kSegBias) << 32) | (kSegBias - (unsigned)cap);
+}
+// Position in the pair array of the claim that read (lo, hi) from a packed counter, or -1 if the segment (or the
+// array) is full.  (Counters that were not prepared for this problem may hold anything: whatever comes out is
+// either -1 or inside the array.)
+__device__ __forceinline__ int packed_position(unsigned lo, unsigned hi, int pair_cap) {
+    const unsigned at = hi + lo;
+    return ((int)lo >= 0 && at < (unsigned)pair_cap) ? (int)at : -1;
+}
 
-// Where claim number `pos` of segment i0 lies in the pair array, or -1 if the segment (or the array) is full
+// Where claim number `pos` of segment i0 lies when every segment holds pair_cap pairs, or -1 if the segment is full
 // (compared as unsigned: counters that were not prepared for this problem may hold anything, and a negative
 // position must not become an address).
-__device__ __forceinline__ int fixed_position(const SegTable &segs, int pair_cap, int i0, int pos) {
-    if (segs.tab != nullptr) {
-        const int2 seg = segs.tab[i0];
-        const int at = seg.x + pos;
-        return ((unsigned)pos < (unsigned)seg.y && (unsigned)at < (unsigned)pair_cap) ? at : -1;
-    }
+__device__ __forceinline__ int fixed_position(int pair_cap, int i0, int pos) {
     return (unsigned)pos < (unsigned)pair_cap ? i0 * pair_cap + pos : -1;
 }
 
@@ -131,9 +142,14 @@ __device__ __forceinline__ int claim_pair(const int *__restrict__ chunk_prefix, 
         const int pos = atomicAdd(cursor + i0, 1) + chunk_prefix[i0 >> kScanChunkBits];
         return (unsigned)pos < (unsigned)pair_cap ? pos : -1;
     }
-    // fixed segments per (texel, replica), of pair_cap pairs each or sized by the geometry: cursor counts from zero
     const int i0 = texel * kFixedReplicas + (rep & (kFixedReplicas - 1));
-    return fixed_position(segs, pair_cap, i0, atomicAdd(cursor + i0, 1));      // (the table entry travels with the atomic)
+    if (segs.tab != nullptr) {
+        // segments sized by the geometry: packed counters
+        const unsigned long long old = atomicAdd(reinterpret_cast<unsigned long long *>(cursor) + i0, 1ull);
+        return packed_position((unsigned)old, (unsigned)(old >> 32), pair_cap);
+    }
+    // fixed segments per (texel, replica) of pair_cap pairs each: cursor counts from zero
+    return fixed_position(pair_cap, i0, atomicAdd(cursor + i0, 1));
 }
 
 // Relative slack of the cheap field-of-view test.  A sample is dropped early only if its
@@ -396,17 +412,27 @@ __device__ __forceinline__ void phase_a_samples(const KParams &k, const WaveLds 
             const int rep = replica_of(cellxy & 0xffff, cellxy >> 16);
             const bool counted = chunk_prefix != nullptr;
             const int i0 = counted ? tx.x * kReplicas + rep : tx.x * kFixedReplicas + (rep & (kFixedReplicas - 1));
-            int pos = 0;
-            if (keep && run_lead == lane) pos = atomicAdd(cursor + i0, run_len);
-            pos = __shfl(pos, run_lead, kWave) + (lane - run_lead);
-            if (keep) {
-                if (counted) {
-                    pos += chunk_prefix[i0 >> kScanChunkBits];
-                    pos = (unsigned)pos < (unsigned)pair_cap ? pos : -1;
-                } else {
-                    pos = fixed_position(segs, pair_cap, i0, pos);
+            if (segs.tab != nullptr) {
+                // packed counters: both words of the lead's answer go round
+                unsigned long long word = 0;
+                if (keep && run_lead == lane)
+                    word = atomicAdd(reinterpret_cast<unsigned long long *>(cursor) + i0, (unsigned long long)run_len);
+                const unsigned lo_w = (unsigned)__shfl((int)(unsigned)word, run_lead, kWave) + (unsigned)(lane - run_lead);
+                const unsigned hi_w = (unsigned)__shfl((int)(unsigned)(word >> 32), run_lead, kWave);
+                if (keep) reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = packed_position(lo_w, hi_w, pair_cap);
+            } else {
+                int pos = 0;
+                if (keep && run_lead == lane) pos = atomicAdd(cursor + i0, run_len);
+                pos = __shfl(pos, run_lead, kWave) + (lane - run_lead);
+                if (keep) {
+                    if (counted) {
+                        pos += chunk_prefix[i0 >> kScanChunkBits];
+                        pos = (unsigned)pos < (unsigned)pair_cap ? pos : -1;
+                    } else {
+                        pos = fixed_position(pair_cap, i0, pos);
+                    }
+                    reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
                 }
-                reinterpret_cast<int *>(L.lst + (size_t)at * ENTRY_F4)[3] = pos;
             }
         }
         if (active && lane == lo) {
