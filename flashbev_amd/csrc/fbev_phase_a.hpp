@@ -114,6 +114,13 @@ constexpr unsigned kSegBias = 0x80000000u;
 __host__ __device__ __forceinline__ unsigned long long packed_counter(int start, int cap) {
     return ((unsigned long long)((unsigned)start + (unsigned)cap - kSegBias) << 32) | (kSegBias - (unsigned)cap);
 }
+// The addend of a single claim on a packed counter, made where it is used: as a constant the compiler would hold
+// the pair of registers from the kernel's start to its end, and the cell pass's fp16 instantiation has none to spare.
+__device__ __forceinline__ unsigned long long fresh_one() {
+    unsigned long long one = 1ull;
+    asm volatile("" : "+v"(one));
+    return one;
+}
 // Position in the pair array of the claim that read (lo, hi) from a packed counter, or -1 if the segment (or the
 // array) is full.  (Counters that were not prepared for this problem may hold anything: whatever comes out is
 // either -1 or inside the array.)
@@ -145,7 +152,7 @@ __device__ __forceinline__ int claim_pair(const int *__restrict__ chunk_prefix, 
     const int i0 = texel * kFixedReplicas + (rep & (kFixedReplicas - 1));
     if (segs.tab != nullptr) {
         // segments sized by the geometry: packed counters
-        const unsigned long long old = atomicAdd(reinterpret_cast<unsigned long long *>(cursor) + i0, 1ull);
+        const unsigned long long old = atomicAdd(reinterpret_cast<unsigned long long *>(cursor) + i0, fresh_one());
         return packed_position((unsigned)old, (unsigned)(old >> 32), pair_cap);
     }
     // fixed segments per (texel, replica) of pair_cap pairs each: cursor counts from zero
