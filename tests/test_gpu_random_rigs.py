@@ -5,7 +5,8 @@ wrap around the image, tiles that straddle the field of view -- the cases the ke
 rejection and the column backward's culling must get right.  Everything is compared with the C
 oracle: masks and indices bit for bit, outputs and gradients within 1e-5 + 1e-4 |ref|, in fp32, fp16
 and bf16 inputs by turns; the forward on cached geometry must repeat the forward's bits, and every
-backward algorithm and workspace kind must agree with the oracle."""
+backward algorithm, workspace kind and layout, with and without the forward's sample store, must agree with the
+oracle."""
 import dataclasses
 import math
 
@@ -80,7 +81,7 @@ def test_random_rig(seed):
     assert torch.equal(got, out) and torch.equal(got_cnt, cnt)
     want_dd, want_df = U.oracle_backward(x, w, dist, thr)
     for mode in ("scatter", "gather", "gather_counted", "columns", "columns_acc", "gather_overwrite",
-                 "persistent_overwrite"):
+                 "persistent_overwrite", "sized_overwrite", "stored", "stored_sized_overwrite"):
         dd, df = U.capi_backward(x, w, dist, thr, mode=mode)
         for got, r, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
             bad, maxabs, ratio = U.violations(got.cpu().numpy(), r)
@@ -125,7 +126,8 @@ def test_random_shapes(seed):
     got, got_cnt = U.capi_forward_cached(x, w, dist, cache, thr, with_count=True)
     assert torch.equal(got, out) and torch.equal(got_cnt, cnt)
     want_dd, want_df = U.oracle_backward(x, w, dist, thr)
-    for mode in ("gather", "gather_counted", "persistent_overwrite", "columns", "scatter"):
+    for mode in ("gather", "gather_counted", "persistent_overwrite", "sized_overwrite", "stored_persistent_overwrite",
+                 "stored_sized", "columns", "scatter"):
         dd, df = U.capi_backward(x, w, dist, thr, mode=mode)
         for got, r, what in ((df, want_df, "d_feats"), (dd, want_dd, "d_depth")):
             bad, maxabs, ratio = U.violations(got.cpu().numpy(), r, rtol=3e-4, atol=3e-5)
