@@ -20,7 +20,9 @@ parameters, tools/config/config.yaml:29).  The single JSON line printed on stdou
                         bytes / the summed mean durations of its kernels, measured with HIP
                         events the library records around every one of its launches over a
                         second run of the same K steps, against the 8 TB/s HBM3E peak;
-                        "kernels" lists every kernel's mean duration and launch count
+                        "kernels" lists every kernel's mean duration and launch count;
+                        "gather_path" is the second ceiling of these kernels: the rows their gathers ask
+                        of the vector L1s (four per kept sample) against 256 CUs x 64 B x 2.4 GHz
   other_workloads       the height-bin sweep (forward, 4 / 8 / 12 / 16 bins), the high-resolution inference and
                         the training-size configurations timed in the same run (forward; forward and
                         backward), with their compulsory bytes and fraction of the HBM peak (which means
@@ -51,6 +53,16 @@ from flashbev_amd.flash_bevpool import voxel_geometry  # noqa: E402
 from flashbev_amd.workloads import WORKLOADS, algorithmic_bytes, make_inputs  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+# What the vector L1s can hand to the lanes: 256 CUs x 64 bytes per clock x 2.4 GHz.  The second ceiling of a gather
+# pass: every kept sample asks for four rows, whatever cache they come from.
+L1_PEAK_GBS = 256 * 64 * 2.4
+
+
+def gather_path(kept: int, channels: int, row_elem_bytes: int, ms: float):
+    """Bytes the four row gathers per kept sample ask of the L1s, and the rate against what the L1s deliver."""
+    nbytes = kept * 4 * channels * row_elem_bytes
+    return {"bytes": nbytes, "achieved": nbytes / ms / 1e6, "peak": L1_PEAK_GBS, "unit": "GB/s",
+            "frac": nbytes / ms / 1e6 / L1_PEAK_GBS}
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same
 # counters read for a 256 MiB copy: kept beside the profile summaries they come from, keyed
 # "workload/depth model/backward mode".  Anything the counters were not collected on reports null.
@@ -383,6 +395,7 @@ def other_workloads(steps: int, warmup: int, backward_mode: int):
             rec["forward_cached_geometry"] = {"ms": c_ms, "frac_hbm": fb / c_ms / 1e6 / HBM_PEAK_GBS, "cache_bytes": c_bytes}
         r.forward()
         rec["kept_samples"] = int(r.counts.sum().item())
+        rec["forward"]["gather_path"] = gather_path(rec["kept_samples"], w.channels, 4 if w.dtype == torch.float32 else 2, f_ms)
         if with_backward and r.workspace is not None:
             rec["backward_workspace"] = {"bytes": r.workspace.numel(),
                                          "layout": "segments sized by the geometry" if r.workspace_layout == 2
@@ -580,6 +593,11 @@ def main():
                      "traffic_kernels": traffic.get("kernels") if traffic else None,
                      "algorithmic_bytes": k_bytes,
                      "kernel_ms": k_ms,
+                     # the other ceiling: the rows the gathers of each kernel ask of the L1s (feature rows in the
+                     # forward and the cell pass, fp32 grad_out rows in the texel pass) against the L1s' rate
+                     "gather_path": {k: gather_path(kept, w.channels, 4 if "texel" in k else es,
+                                                    kernels[k]["mean_us"] * kernels[k]["calls_per_step"] / 1e3)
+                                     for k in kernels if any(t in k for t in ("forward", "cells", "texel"))},
                      "forward": {"algorithmic_bytes": fb, "kernel_ms": fwd_k_ms,
                                  "frac": fb / fwd_k_ms / 1e6 / HBM_PEAK_GBS if fwd_k_ms else None}},
     }
