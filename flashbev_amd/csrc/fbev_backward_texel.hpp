@@ -43,7 +43,9 @@ struct Persist {
     SegTable segs;
 };
 
-template <int VEC, int WAVES>
+// NARROW: grad_out is smaller than 4 GiB, so a row is addressed by a 32-bit byte offset from the tensor's uniform base
+// (one add per gather instead of a 64-bit shift-add: a sixth of the pass's vector instructions).
+template <int VEC, int WAVES, bool NARROW>
 __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
     KParams k, const float *__restrict__ grad_out, const int *__restrict__ chunk_prefix,
     const int *__restrict__ seg_end, const Pair *__restrict__ pairs, int pair_cap, float *__restrict__ d_depth,
@@ -180,12 +182,18 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
         __syncthreads();
     }
     constexpr int kOutShift = VEC > 1 ? 4 : 2;
-    const unsigned out_units = (unsigned)(VEC > 1 ? k.C / 4 : k.C);
+    const unsigned out_units = NARROW ? (unsigned)k.C * 4u : (unsigned)(VEC > 1 ? k.C / 4 : k.C);
     const char *gbytes = reinterpret_cast<const char *>(grad_out);
+    unsigned ch_bytes = 0;      // (set per channel pass: where the lane's channels start in a row)
+    auto row_at = [&](unsigned row) {
+        return NARROW ? reinterpret_cast<const float *>(gbytes + (row + ch_bytes))
+                      : reinterpret_cast<const float *>(gbytes + ((size_t)row << kOutShift)) + (ch_bytes >> 2);
+    };
     for (int c0 = 0; c0 < k.C; c0 += span) {
         const int ch = c0 + lir * VEC;
         const bool on = worker_lane && ch < k.C;
-        const int ch_eff = on ? ch : 0, wslot_eff = min(wslot, wpw - 1);
+        const int wslot_eff = min(wslot, wpw - 1);
+        ch_bytes = on ? (unsigned)ch * 4u : 0u;
         float acc[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
@@ -226,7 +234,8 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
             else if (o == 1) cw = fu ? w10 + (fv ? 0.0f : w11) : 0.0f;
             else if (o == 2) cw = fv ? w01 + (fu ? 0.0f : w11) : 0.0f;
             else cw = (fu && fv) ? w11 : 0.0f;
-            // where the pair's grad_out row starts, in units of 16 bytes (one float off the vector path)
+            // where the pair's grad_out row starts: in bytes, or (a tensor of 4 GiB and more) in units of 16 bytes
+            // (one float off the vector path)
             const unsigned my_row = valid ? (unsigned)(word >> bin_bits) * out_units : 0u;
             const float my_coef = valid ? pr.y * cw : 0.0f;
             if (c0 == 0 && valid) {
@@ -273,7 +282,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
                 for (int q = 0; q < UNR; ++q) {
                     const float2 rc = stage[i + q * wpw + wslot_eff];
                     coefs[q] = rc.y;
-                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g[q]);
+                    VecLoad<float, VEC>::ld(row_at((unsigned)__float_as_int(rc.x)), g[q]);
                 }
 #pragma unroll
                 for (int q = 0; q < UNR; ++q)
@@ -290,7 +299,7 @@ __global__ __launch_bounds__(kWave *WAVES) void fbev_backward_texel_kernel(
                     const int want = full + q * wpw + wslot_eff;
                     const float2 rc = stage[min(want, n_lead - 1)];
                     coefs[q] = want < n_lead ? rc.y : 0.0f;
-                    VecLoad<float, VEC>::ld(reinterpret_cast<const float *>(gbytes + ((size_t)(unsigned)__float_as_int(rc.x) << kOutShift)) + ch_eff, g[q]);
+                    VecLoad<float, VEC>::ld(row_at((unsigned)__float_as_int(rc.x)), g[q]);
                 }
 #pragma unroll
                 for (int q = 0; q < UNR; ++q)

@@ -692,14 +692,22 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
         hipLaunchKernelGGL(kernel, tgrid, tblock, lds, st, pl.k, grad_out, prefix_arg, cursor, pairs, cap_arg, d_depth, d_feats,
                            lpr, from_pairs, accumulate ? 0 : 1, ps);
     };
+    // (rows of a grad_out below 4 GiB are addressed with 32-bit byte offsets)
+    const bool narrow = (uint64_t)p->batch * p->grid_y * p->grid_x * p->channels * sizeof(float) < (1ull << 32);
+    auto launch_waves = [&](auto vec_tag, auto narrow_tag) {
+        constexpr int V = decltype(vec_tag)::value;
+        constexpr bool N = decltype(narrow_tag)::value;
+        if (texel_waves == 1) launch(fbev_backward_texel_kernel<V, 1, N>);
+        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<V, 2, N>);
+        else launch(fbev_backward_texel_kernel<V, kWavesPerBlock, N>);
+    };
+    using std::integral_constant;
     if (vec4) {
-        if (texel_waves == 1) launch(fbev_backward_texel_kernel<4, 1>);
-        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<4, 2>);
-        else launch(fbev_backward_texel_kernel<4, kWavesPerBlock>);
+        if (narrow) launch_waves(integral_constant<int, 4>{}, integral_constant<bool, true>{});
+        else launch_waves(integral_constant<int, 4>{}, integral_constant<bool, false>{});
     } else {
-        if (texel_waves == 1) launch(fbev_backward_texel_kernel<1, 1>);
-        else if (texel_waves == 2) launch(fbev_backward_texel_kernel<1, 2>);
-        else launch(fbev_backward_texel_kernel<1, kWavesPerBlock>);
+        if (narrow) launch_waves(integral_constant<int, 1>{}, integral_constant<bool, true>{});
+        else launch_waves(integral_constant<int, 1>{}, integral_constant<bool, false>{});
     }
     return hipGetLastError() == hipSuccess ? FBEV_OK : FBEV_ERR_LAUNCH;
 }

@@ -319,6 +319,28 @@ def test_fixed_segments_overflow_falls_back_to_atomics(dist):
     check_all(w, x, dist, thr=0.0, modes=("sized", "sized_overwrite"), bwd_tol=(3e-4, 3e-5))
 
 
+def test_grad_out_of_four_gib_takes_the_wide_row_addresses():
+    """The texel pass addresses a grad_out row with a 32-bit byte offset while the tensor stays below 4 GiB, which
+    every benchmark configuration does, and with 64-bit arithmetic from there on.  A 1024 x 2048 grid with 512
+    channels is exactly 4 GiB: the inverse map must agree with the atomic scatter, which never gathers a row (an
+    address that wrapped would show as differences of the size of the values)."""
+    w = dataclasses.replace(WORKLOADS["cfg2_surround"], batch=1, channels=512, grid_size=(2048, 1024, 1))
+    x = make_inputs(w, "parametric", device="cuda", with_grad_out=False)
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    x["grad_out"] = torch.randn(1, 1024, 2048, 512, device="cuda", generator=gen)
+    assert x["grad_out"].numel() * 4 == 1 << 32
+    want_dd, want_df = U.capi_backward(x, w, 1, 1e-6, mode="scatter_overwrite")
+    assert float(want_df.abs().max()) > 0.1
+    for mode in ("gather_overwrite", "persistent_overwrite"):
+        dd, df = U.capi_backward(x, w, 1, 1e-6, mode=mode)
+        for got, ref in ((df, want_df), (dd, want_dd)):
+            err = (got - ref).abs()
+            assert bool((err <= 5e-5 + 5e-4 * ref.abs()).all()), (mode, float(err.max()))
+        del dd, df
+    del x
+    torch.cuda.empty_cache()
+
+
 def test_the_reference_calibration_fixture():
     """The reference's own six-camera nuScenes calibration (its inputs/calib_nuscenes.json, kept as
     data under tests/golden/): masks, indices and fractions bit for bit, values within tolerance,
