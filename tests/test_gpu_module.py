@@ -363,6 +363,65 @@ def test_operator_backward_variants_agree(monkeypatch, env):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("layout,seed", [("auto", 1), ("auto", 2), ("sized", 3), ("fixed", 4)])
+def test_operator_over_a_changing_sequence_of_shapes_and_matrices(monkeypatch, layout, seed):
+    """What the operator keeps between calls -- workspaces per shape, their layout and the matrices a sized one was
+    counted for, the sample store of a forward -- under a random sequence of differentiated calls over four shapes
+    and input types: matrices that stay, are scaled in place or are replaced, thresholds that change, forwards whose
+    backward never runs, leaves that want no gradient.  Every gradient against the C ABI's atomic scatter on the
+    same inputs (fp32 leaves: 5e-5 + 5e-4 |ref|, two summation orders of fp32; half-precision leaves receive their
+    gradient rounded to their type)."""
+    import dataclasses
+    from flashbev_amd import flash_bevpool
+    from flashbev_amd.workloads import WORKLOADS, make_inputs
+    from tests.test_gpu_random_rigs import random_pose
+
+    monkeypatch.setenv("FLASHBEV_WORKSPACE_LAYOUT", layout)
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(4):
+        n_cams, batch = int(rng.integers(1, 7)), int(rng.integers(1, 3))
+        w = dataclasses.replace(WORKLOADS["cfg1_tiny"], batch=batch, yaws=tuple([0.0] * n_cams),
+                                channels=int(rng.choice([8, 20, 64, 80])),
+                                feat_hw=(int(rng.integers(4, 20)), int(rng.integers(6, 44))),
+                                grid_size=(int(rng.integers(16, 120)), int(rng.integers(16, 120)), int(rng.integers(1, 13))),
+                                depth_bins=int(rng.integers(3, 40)))
+        dist = int(rng.integers(0, 3))
+        x = make_inputs(w, "categorical" if dist == 2 else "parametric", device="cuda", with_grad_out=True)
+        dtype = (torch.float32, torch.float16, torch.bfloat16)[int(rng.integers(0, 3))]
+        for name in ("image_feats", "depth_params"):
+            x[name] = x[name].to(dtype).contiguous()
+        shapes.append((w, dist, x))
+    checked = 0
+    for it in range(40):
+        w, dist, x = shapes[int(rng.integers(0, len(shapes)))]
+        r = rng.random()
+        if r < 0.25:
+            P = np.stack([[random_pose(rng) for _ in range(w.num_cams)] for _ in range(w.batch)]).astype(np.float32)
+            x["projection_matrices"] = torch.from_numpy(P).cuda().contiguous()
+        elif r < 0.4:
+            x["projection_matrices"].mul_(1.0 + 1e-3 * float(rng.random()))
+        thr = float(rng.choice([0.0, 1e-6, 1e-3]))
+        feats = x["image_feats"].clone().requires_grad_(bool(rng.random() < 0.8))
+        depth = x["depth_params"].clone().requires_grad_(bool(rng.random() < 0.8) or not feats.requires_grad)
+        out = flash_bevpool(feats, depth, x["projection_matrices"], x["feature_size"], x["image_size"], x["roi_range"],
+                            x["grid_size"], depth_distribution=dist, epsilon=1e-6, depth_weight_threshold=thr,
+                            depth_range=w.depth_range if dist == 2 else None)
+        if rng.random() < 0.2:
+            continue                                    # a forward whose backward never runs
+        out.backward(x["grad_out"])
+        want_dd, want_df = U.capi_backward(x, w, dist, thr, mode="scatter_overwrite")
+        for got, ref, name in ((feats.grad, want_df, "d_feats"), (depth.grad, want_dd, "d_depth")):
+            if got is None:
+                continue
+            tol = 5e-5 + 5e-4 * ref.abs() if got.dtype == torch.float32 else 2e-3 + 2e-2 * ref.abs()
+            err = (got.float() - ref).abs()
+            assert bool((err <= tol).all()), (it, name, layout, float(err.max()), int((err > tol).sum()))
+            checked += 1
+    assert checked > 30
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("extra", [["--num-height-bins", "4", "8"], ["--num-cameras-list", "1", "6", "--module"]])
 def test_latency_sweep_harness_runs_and_keeps_the_reference_record_layout(extra, tmp_path):
     """profile_latency.run on a two-point sweep (a small grid, few timed calls): one record per point
