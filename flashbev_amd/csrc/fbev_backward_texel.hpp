@@ -18,9 +18,12 @@ namespace {
 constexpr int kTexelMaxSplit = 8;
 constexpr int kTexelSplitBelow = 16384;     // texels * blocks per texel stay below this (400x400x12 grid on 4224 texels: 1 / 3 / 7 blocks per texel 107 / 101 / 127 us)
 constexpr int kTexelPart = 128;
-constexpr int kTexelOneWaveBelow = 100;      // possible samples per texel below which a block is one wavefront ...
-constexpr int kTexelManyTexels = 50000;      // ... or three times that when there are this many texels
-constexpr int kTexelTwoWavesBelow = 450;     // below which it is two wavefronts; four from there on
+// Wavefronts per texel block, chosen from the samples a texel could get if every one were kept ("possible"), counted
+// twice where about twice as many are kept (categorical depth, or no weight threshold):
+constexpr int kTexelOneWaveBelow = 200;      // one wavefront below this ...
+constexpr int kTexelManyTexels = 50000;      // ... or, with this many texels, below kTexelOneWaveManyBelow possible samples
+constexpr int kTexelOneWaveManyBelow = 300;
+constexpr int kTexelTwoWavesBelow = 800;     // two wavefronts below this; four from there on
 constexpr int kTexelSegs = 4 * kFixedReplicas;   // lists of a texel with fixed segments: 4 first corners x replicas
 
 // What a persistent workspace adds to the fixed-segment layout, so that a call needs no zero-fill

@@ -668,13 +668,18 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     // One, two or four wavefronts per texel.  A texel's block is a chain of dependent loads (list bounds,
     // pairs, grad_out rows); small blocks fit the machine in fewer generations, large ones shorten the
     // chain of a long list.  What is known here is only how many samples a texel could get if every one were
-    // kept.  Measured (us for 1 / 2 / 4 wavefronts; Laplace, then the categorical model, which keeps twice
-    // as many): 23 possible samples per texel 8 / 9 / 11; 186 per texel and 4224 texels 20 / 19 / 23 and
-    // 39 / 30 / 31; 186 per texel and 67 584 texels 125 / 154 / 239 and 256 / 274 / 365; 454 per texel
-    // 38 / 29 / 29 and 80 / 60 / 52; 909 per texel 493 / 426 / 431; 2727 per texel 352 / 209 / 124.
+    // kept, and that the categorical model, or a threshold of zero, keeps about twice as many as the parametric
+    // models under a threshold.  Measured (us for 1 / 2 / 4 wavefronts; Laplace, then the categorical model):
+    // 23 possible samples per texel 8.2 / 8.9 / 10.4 and 8.2 / 8.7 / 10.1; 186 per texel and 4224 texels
+    // 17.3 / 18.2 / 23.5 and 32.6 / 26.1 / 30.4; 227: 21.6 / 20.5 / 24.8 and 41.0 / 33.5 / 34.5; 454: 33.0 / 26.1 / 28.2
+    // and 64.9 / 49.4 / 46.8; 681: 39.7 / 30.9 / 31.5 and 90.2 / 65.9 / 59.5; 909: 44.5 / 33.8 / 33.6 and
+    // 114.5 / 82.4 / 71.2; 1818: 102.8 / 70.0 / 53.3 and 287.2 / 204.4 / 133.5; 186 per texel and 67 584 texels
+    // 125 / 154 / 239 and 256 / 274 / 365.
     const uint64_t per_texel = fbev_backward_max_pairs(p) / (uint64_t)texels;
-    const int texel_waves = (per_texel < kTexelOneWaveBelow || (texels >= kTexelManyTexels && per_texel < 3 * kTexelOneWaveBelow)) ? 1
-                            : (per_texel < kTexelTwoWavesBelow ? 2 : kWavesPerBlock);
+    const bool keeps_most = p->depth_distribution == FBEV_CATEGORICAL || !(p->depth_weight_threshold > 0.0f);
+    const uint64_t expected = per_texel * (keeps_most ? 2 : 1);
+    const int texel_waves = (expected < kTexelOneWaveBelow || (texels >= kTexelManyTexels && per_texel < kTexelOneWaveManyBelow)) ? 1
+                            : (expected < kTexelTwoWavesBelow ? 2 : kWavesPerBlock);
     const int nw = (kWave / lpr) * texel_waves;
     // the depth gradient rides on the pairs exactly when the cell pass folds it in (one channel pass
     // and room for the depth bin in a pair's first word)
