@@ -20,10 +20,13 @@ constexpr int kTexelSplitBelow = 16384;     // texels * blocks per texel stay be
 constexpr int kTexelPart = 128;
 // Wavefronts per texel block, chosen from the samples a texel could get if every one were kept ("possible"), counted
 // twice where about twice as many are kept (categorical depth, or no weight threshold):
-constexpr int kTexelOneWaveBelow = 200;      // one wavefront below this ...
-constexpr int kTexelManyTexels = 50000;      // ... or, with this many texels, below kTexelOneWaveManyBelow possible samples
-constexpr int kTexelOneWaveManyBelow = 300;
-constexpr int kTexelTwoWavesBelow = 800;     // two wavefronts below this; four from there on
+constexpr int kTexelOneWaveBelow = 200;      // one wavefront below this,
+constexpr int kTexelTwoWavesBelow = 800;     // two below this, four from there on;
+// and one instead of two when two would make more wavefronts than eight times what the machine holds at once
+// (256 CUs x 4 SIMDs x 6): the blocks then run in many generations anyway, and what a second wavefront per block adds
+// is its share of the set-up, not a shorter chain.  (Four are kept: at the training size two per texel are 3 % faster
+// but put twice the texels in flight per die, more than its L2 holds grad_out rows for: 541 instead of 382 MB from HBM.)
+constexpr long long kTexelWavesAtOnce = 8ll * 256 * 4 * 6;
 constexpr int kTexelSegs = 4 * kFixedReplicas;   // lists of a texel with fixed segments: 4 first corners x replicas
 
 // What a persistent workspace adds to the fixed-segment layout, so that a call needs no zero-fill

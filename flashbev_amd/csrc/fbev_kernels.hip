@@ -673,13 +673,15 @@ int backward_gather_impl(const fbev_problem *p, const float *grad_out, const voi
     // 23 possible samples per texel 8.2 / 8.9 / 10.4 and 8.2 / 8.7 / 10.1; 186 per texel and 4224 texels
     // 17.3 / 18.2 / 23.5 and 32.6 / 26.1 / 30.4; 227: 21.6 / 20.5 / 24.8 and 41.0 / 33.5 / 34.5; 454: 33.0 / 26.1 / 28.2
     // and 64.9 / 49.4 / 46.8; 681: 39.7 / 30.9 / 31.5 and 90.2 / 65.9 / 59.5; 909: 44.5 / 33.8 / 33.6 and
-    // 114.5 / 82.4 / 71.2; 1818: 102.8 / 70.0 / 53.3 and 287.2 / 204.4 / 133.5; 186 per texel and 67 584 texels
-    // 125 / 154 / 239 and 256 / 274 / 365.
+    // 114.5 / 82.4 / 71.2; 1818: 102.8 / 70.0 / 53.3 and 287.2 / 204.4 / 133.5.  With more texels: 186 per texel on
+    // 33 792 texels 56.8 / 80.3 / 135.1 and 94.0 / 113.2 / 163.6, on 67 584 texels 111.9 / 160.4 / 266.4 and
+    // 210.6 / 247.6 / 349.0; 909 per texel on 8448 texels 124.7 / 92.0 / 88.1 and 218.9 / 160.2 / 152.3, on 33 792
+    // texels 390.6 / 337.6 / 344.1 and 655.5 / 554.4 / 567.4.
     const uint64_t per_texel = fbev_backward_max_pairs(p) / (uint64_t)texels;
     const bool keeps_most = p->depth_distribution == FBEV_CATEGORICAL || !(p->depth_weight_threshold > 0.0f);
     const uint64_t expected = per_texel * (keeps_most ? 2 : 1);
-    const int texel_waves = (expected < kTexelOneWaveBelow || (texels >= kTexelManyTexels && per_texel < kTexelOneWaveManyBelow)) ? 1
-                            : (expected < kTexelTwoWavesBelow ? 2 : kWavesPerBlock);
+    int texel_waves = expected < kTexelOneWaveBelow ? 1 : (expected < kTexelTwoWavesBelow ? 2 : kWavesPerBlock);
+    if (texel_waves == 2 && texels * texel_waves > kTexelWavesAtOnce) texel_waves = 1;
     const int nw = (kWave / lpr) * texel_waves;
     // the depth gradient rides on the pairs exactly when the cell pass folds it in (one channel pass
     // and room for the depth bin in a pair's first word)
